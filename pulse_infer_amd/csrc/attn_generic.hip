@@ -9,7 +9,10 @@
 // query head h reads kv head h / (nq / nkv) (paged_attention.cu:61-70).
 //
 // With `gate` every head's output is multiplied by sigmoid(gate[token, head]) before it is stored (an output gate
-// whose logits another product left, one a token and head, `gate_stride` elements from row to row).
+// whose logits another product left, one a token and head, `gate_stride` elements from row to row); with
+// `gate_width` > 0 there is a logit for each of the first `gate_width` channels of every head instead
+// (gate[token, head * gate_width + channel]).  `softcap` > 0 bounds the scaled scores, s <- cap * tanh(s / cap).
+// `sink` (float32, one a query head) adds exp(sink[h]) to the softmax's denominator: a term without key or value.
 //
 // This is the kernel of the true 32-bit path and the fallback for sizes that the
 // matrix-core kernels refuse.
@@ -27,6 +30,9 @@ struct AttnArgs {
     int page_size, num_pages, bt_width;
     float scale;
     int window;  // 0: all keys
+    float cap;   // > 0: a score s becomes cap * tanh(s / cap); 0: scores as they are
+    int gate_per_channel;   // 0: one gate logit a head; 1: one a channel (gate [T, nq * gate_width])
+    int gate_width;         // channels of a head that have a gate logit (the others are stored ungated)
 };
 
 template <typename TX, typename TC>
@@ -36,7 +42,8 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const TX* __restrict__
                                                           const int* __restrict__ positions,
                                                           const int* __restrict__ token_entry,
                                                           const int* __restrict__ block_table,
-                                                          const TX* __restrict__ gate, int64_t gate_stride, AttnArgs a) {
+                                                          const TX* __restrict__ gate, int64_t gate_stride,
+                                                          const float* __restrict__ sink, AttnArgs a) {
     extern __shared__ long long lds[];
     long long* v_s = lds;                                         // [64] value offsets of a tile's keys
     float* p_s = reinterpret_cast<float*>(lds + PULSE_WAVE);      // [64] a tile's probabilities
@@ -74,7 +81,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const TX* __restrict__
                 const TC* krow = kcache + (pg * a.page_size + slot) * d;
                 float dot = 0.f;
                 for (int e = 0; e < d; ++e) dot = fmaf(q_s[e], to_f32<TC>(krow[e]), dot);
-                s = dot;
+                s = a.cap > 0.f ? a.cap * tanhf(dot / a.cap) : dot;
                 vbase = pg * d * a.page_size + slot;
             }
         }
@@ -105,12 +112,27 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const TX* __restrict__
     }
 
     TX* orow = out + static_cast<int64_t>(t) * a.o_stride + static_cast<int64_t>(h) * d;
+    // a sink is one more term of the softmax's denominator, exp(sink[h]), with no key and no value
+    if (sink) {
+        const float sk = sink[h];
+        if (m == -INFINITY) { l = 1.f; }
+        else if (sk > m) { l = l * expf(m - sk) + 1.f; const float f = expf(m - sk);
+#pragma unroll
+            for (int r = 0; r < MAX_ACC; ++r) acc[r] *= f; }
+        else l += expf(sk - m);
+    }
     float inv_l = l > 0.f ? 1.0f / l : 0.f;
-    if (gate) inv_l *= 1.0f / (1.0f + expf(-to_f32<TX>(gate[static_cast<int64_t>(t) * gate_stride + h])));
+    const TX* grow = gate ? gate + static_cast<int64_t>(t) * gate_stride : nullptr;
+    if (grow && !a.gate_per_channel) inv_l *= 1.0f / (1.0f + expf(-to_f32<TX>(grow[h])));
 #pragma unroll
     for (int r = 0; r < MAX_ACC; ++r) {
         const int e = lane + r * PULSE_WAVE;
-        if (e < d) orow[e] = from_f32<TX>(acc[r] * inv_l);
+        if (e < d) {
+            float v = acc[r] * inv_l;
+            if (grow && a.gate_per_channel && e < a.gate_width)
+                v *= 1.0f / (1.0f + expf(-to_f32<TX>(grow[static_cast<int64_t>(h) * a.gate_width + e])));
+            orow[e] = from_f32<TX>(v);
+        }
     }
 }
 
@@ -120,7 +142,8 @@ extern "C" int pulse_attn_generic(const void* q, int64_t q_stride, void* out, in
                                   const void* kcache, const void* vcache, int c_dtype, const int* positions,
                                   const int* token_entry, const int* block_table, int bt_width, int tokens, int nq,
                                   int nkv, int d, int page_size, int num_pages, float scale, int window,
-                                  const void* gate, int64_t gate_stride, hipStream_t stream) {
+                                  const void* gate, int64_t gate_stride, int gate_width, const float* sink,
+                                  float softcap, hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && nq > 0 && nkv > 0 && d > 0, "attn_generic: bad sizes");
     PULSE_REQUIRE(nq % nkv == 0, "attn_generic: %d query heads are not a multiple of %d kv heads", nq, nkv);
     PULSE_REQUIRE(d <= PULSE_WAVE * MAX_ACC, "attn_generic: head_dim %d exceeds %d", d, PULSE_WAVE * MAX_ACC);
@@ -131,17 +154,21 @@ extern "C" int pulse_attn_generic(const void* q, int64_t q_stride, void* out, in
                   "attn_generic: row strides too small");
     PULSE_REQUIRE(pulse_dtype_ok(x_dtype) && pulse_dtype_ok(c_dtype), "attn_generic: bad dtype tag");
     PULSE_REQUIRE(q && out && kcache && vcache && positions && token_entry && block_table, "attn_generic: null pointer");
-    PULSE_REQUIRE(!gate || gate_stride >= nq, "attn_generic: the gate's rows are too short");
+    PULSE_REQUIRE(gate_width >= 0 && gate_width <= d, "attn_generic: %d gated channels of a head of %d", gate_width, d);
+    PULSE_REQUIRE(!gate || gate_stride >= static_cast<int64_t>(nq) * (gate_width ? gate_width : 1),
+                  "attn_generic: the gate's rows are too short");
+    PULSE_REQUIRE(softcap >= 0.f, "attn_generic: a negative score cap");
     if (tokens == 0) return 0;
     AttnArgs a;
     a.nq = nq; a.nkv = nkv; a.d = d; a.q_stride = q_stride; a.o_stride = o_stride;
     a.page_size = page_size; a.num_pages = num_pages; a.bt_width = bt_width; a.scale = scale; a.window = window;
+    a.cap = softcap; a.gate_per_channel = gate_width > 0 ? 1 : 0; a.gate_width = gate_width;
     const size_t lds = static_cast<size_t>(d) * sizeof(float) + PULSE_WAVE * sizeof(float) + PULSE_WAVE * sizeof(long long);
     PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(c_dtype, TC,
         hipLaunchKernelGGL((attn_generic_kernel<TX, TC>), dim3(tokens, nq), dim3(64), lds, stream,
                            static_cast<const TX*>(q), static_cast<TX*>(out), static_cast<const TC*>(kcache),
                            static_cast<const TC*>(vcache), positions, token_entry, block_table,
-                           static_cast<const TX*>(gate), gate_stride, a)));
+                           static_cast<const TX*>(gate), gate_stride, sink, a)));
     PULSE_LAUNCH_CHECK("attn_generic");
     return 0;
 }

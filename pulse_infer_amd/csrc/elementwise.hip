@@ -238,8 +238,14 @@ extern "C" int pulse_residual_add(float* h, const void* delta, int delta_dtype, 
 // slabs of `slab` columns (gate slab, up slab, ...), the layout of a slab-interleaved weight.
 // out[t, i] = silu(g) * u, silu(x) = x / (1 + exp(-x)), product in float32, one rounding.
 // (reference: src/ops/kernels/cuda/silu_kernel.cu:82-97 then mul_kernel.cu:39-46, two roundings)
+// act 0: silu, 1: the tanh form of gelu
+__device__ __forceinline__ float gate_act(float g, int act) {
+    if (act == 1) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.0f + expf(-g));
+}
+
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int slab, int64_t total) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int slab, int64_t total, int act) {
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int64_t t = idx / inter;
@@ -249,13 +255,12 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
     const int ui = slab > 0 ? gi + slab : inter + i;
     const float g = to_f32<T>(row[gi]);
     const float u = to_f32<T>(row[ui]);
-    const float s = g / (1.0f + expf(-g));
-    out[idx] = from_f32<T>(s * u);
+    out[idx] = from_f32<T>(gate_act(g, act) * u);
 }
 
 // Eight outputs a thread with 16-byte accesses, for bfloat16 rows whose sizes allow it.
 __global__ void swiglu_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int inter, int slab,
-                                     int64_t total8) {
+                                     int64_t total8, int act) {
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= total8) return;
     const int per_row = inter / 8;
@@ -273,14 +278,16 @@ __global__ void swiglu_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __re
     for (int j = 0; j < 4; ++j) {
         const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
         const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
-        const float z0 = g0 / (1.0f + expf(-g0)) * u0;
-        const float z1 = g1 / (1.0f + expf(-g1)) * u1;
+        const float z0 = gate_act(g0, act) * u0;
+        const float z1 = gate_act(g1, act) * u1;
         ow[j] = static_cast<uint32_t>(f32_to_bf16(z0)) | (static_cast<uint32_t>(f32_to_bf16(z1)) << 16);
     }
     *reinterpret_cast<uint4*>(out + t * inter + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
-extern "C" int pulse_swiglu(const void* gu, void* out, int dtype, int tokens, int inter, int slab, hipStream_t stream) {
+extern "C" int pulse_swiglu(const void* gu, void* out, int dtype, int tokens, int inter, int slab, int act,
+                            hipStream_t stream) {
+    PULSE_REQUIRE(act == 0 || act == 1, "swiglu: unknown activation %d", act);
     PULSE_REQUIRE(tokens >= 0 && inter > 0 && pulse_dtype_ok(dtype) && gu && out, "swiglu: bad arguments");
     PULSE_REQUIRE(slab >= 0 && (slab == 0 || inter % slab == 0), "swiglu: %d columns do not divide into slabs of %d", inter, slab);
     const int64_t total = static_cast<int64_t>(tokens) * inter;
@@ -292,7 +299,7 @@ extern "C" int pulse_swiglu(const void* gu, void* out, int dtype, int tokens, in
         const int64_t blocks = (total8 + 255) / 256;
         PULSE_REQUIRE(blocks < (1ll << 31), "swiglu: too many elements");
         hipLaunchKernelGGL(swiglu_bf16x8_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
-                           static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), inter, slab, total8);
+                           static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), inter, slab, total8, act);
         PULSE_LAUNCH_CHECK("swiglu");
         return 0;
     }
@@ -300,7 +307,7 @@ extern "C" int pulse_swiglu(const void* gu, void* out, int dtype, int tokens, in
     PULSE_REQUIRE(blocks < (1ll << 31), "swiglu: too many elements");
     PULSE_DISPATCH_DTYPE(dtype, T,
         hipLaunchKernelGGL(swiglu_kernel<T>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
-                           static_cast<const T*>(gu), static_cast<T*>(out), inter, slab, total));
+                           static_cast<const T*>(gu), static_cast<T*>(out), inter, slab, total, act));
     PULSE_LAUNCH_CHECK("swiglu");
     return 0;
 }

@@ -13,6 +13,12 @@
 // pulse_moe_down, a workgroup per token and 64 output columns: out[t, c] = sum_k weight_k * (down row c . act row
 // (t, k)) or weight_k * x[t, c] for an identity expert, added up in the order of choice, in float32.
 // A token's result depends on its own row alone, whatever else the step holds.
+//
+// Variations, as arguments: `score_fn` 1 takes s = sigmoid(z) instead of the softmax; `renorm` 0 leaves the chosen
+// scores as they are.  `in_weight` (gate/up kernels): the expert is fed weight * x, i.e. both products are multiplied
+// by the pair's weight before the activation (the products are linear), and the down kernels are then handed no
+// weight.  `act_kind` 1 is the clamped form g' = min(g, limit), u' = clamp(u, -limit, limit),
+// act = g' * sigmoid(1.702 g') * (u' + 1).
 #include "common.h"
 
 #include <math.h>
@@ -24,7 +30,8 @@ constexpr int ROUTE_PER_LANE = 16;   // router outputs <= 64 * 16
 // One wavefront routes one token: `row` holds its n router logits (in global memory or in LDS).
 template <typename TW>
 __device__ __forceinline__ void route_row(const float* row, const TW* __restrict__ correction, int* __restrict__ idx,
-                                          float* __restrict__ weight, int n, int top, int t, int lane) {
+                                          float* __restrict__ weight, int n, int top, int t, int lane,
+                                          int score_fn, int renorm) {
     float s[ROUTE_PER_LANE], c[ROUTE_PER_LANE];
     float m = -INFINITY;
 #pragma unroll
@@ -38,10 +45,11 @@ __device__ __forceinline__ void route_row(const float* row, const TW* __restrict
 #pragma unroll
     for (int r = 0; r < ROUTE_PER_LANE; ++r) {
         const int j = lane + r * PULSE_WAVE;
-        s[r] = j < n ? expf(s[r] - m) : 0.f;
+        if (score_fn == 1) s[r] = j < n ? 1.0f / (1.0f + expf(-s[r])) : 0.f;
+        else s[r] = j < n ? expf(s[r] - m) : 0.f;
         sum += s[r];
     }
-    sum = wave_sum(sum);
+    sum = score_fn == 1 ? 1.f : wave_sum(sum);
 #pragma unroll
     for (int r = 0; r < ROUTE_PER_LANE; ++r) {
         const int j = lane + r * PULSE_WAVE;
@@ -78,14 +86,16 @@ __device__ __forceinline__ void route_row(const float* row, const TW* __restrict
     }
     if (lane < top) {
         idx[static_cast<int64_t>(t) * top + lane] = mine_idx;
-        weight[static_cast<int64_t>(t) * top + lane] = mine / (total + 1e-20f);
+        weight[static_cast<int64_t>(t) * top + lane] = renorm ? mine / (total + 1e-20f) : mine;
     }
 }
 
 template <typename TW>
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, const TW* __restrict__ correction,
-                                                       int* __restrict__ idx, float* __restrict__ weight, int n, int top) {
-    route_row<TW>(z + static_cast<int64_t>(blockIdx.x) * n, correction, idx, weight, n, top, blockIdx.x, threadIdx.x);
+                                                       int* __restrict__ idx, float* __restrict__ weight, int n, int top,
+                                                       int score_fn, int renorm) {
+    route_row<TW>(z + static_cast<int64_t>(blockIdx.x) * n, correction, idx, weight, n, top, blockIdx.x, threadIdx.x,
+                  score_fn, renorm);
 }
 
 // The router's product and the routing in one: a workgroup a token holds the token's row in LDS, its wavefronts
@@ -94,7 +104,8 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
 template <typename TX, typename TW>
 __global__ __launch_bounds__(1024) void moe_router_kernel(const TX* __restrict__ x, const TW* __restrict__ w,
                                                          const TW* __restrict__ correction, int* __restrict__ idx,
-                                                         float* __restrict__ weight, int hidden, int n, int top) {
+                                                         float* __restrict__ weight, int hidden, int n, int top,
+                                                         int score_fn, int renorm) {
     extern __shared__ float x_s[];          // [hidden] then [n]
     float* z_s = x_s + hidden;
     const int t = blockIdx.x;
@@ -125,14 +136,15 @@ __global__ __launch_bounds__(1024) void moe_router_kernel(const TX* __restrict__
         if (lane == 0) z_s[o] = sum;
     }
     __syncthreads();
-    if (wave == 0) route_row<TW>(z_s, correction, idx, weight, n, top, t, lane);
+    if (wave == 0) route_row<TW>(z_s, correction, idx, weight, n, top, t, lane, score_fn, renorm);
 }
 
 template <typename TX, typename TW>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(const TX* __restrict__ x, const TW* __restrict__ wg,
                                                           const TW* __restrict__ wu, const int* __restrict__ idx,
                                                           TX* __restrict__ act, int hidden, int ff, int experts,
-                                                          int top) {
+                                                          int top, const float* __restrict__ in_weight, int act_kind,
+                                                          float limit) {
     extern __shared__ float x_s[];
     const int a = blockIdx.x;
     const int e = idx[a];
@@ -152,7 +164,15 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const TX* __restrict__
         }
         sg = wave_sum(sg);
         su = wave_sum(su);
-        if (lane == 0) act[static_cast<int64_t>(a) * ff + j] = from_f32<TX>(sg / (1.0f + expf(-sg)) * su);
+        if (in_weight) { sg *= in_weight[a]; su *= in_weight[a]; }
+        float v;
+        if (act_kind == 1) {
+            const float g = fminf(sg, limit), u = fminf(fmaxf(su, -limit), limit);
+            v = g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+        } else {
+            v = sg / (1.0f + expf(-sg)) * su;
+        }
+        if (lane == 0) act[static_cast<int64_t>(a) * ff + j] = from_f32<TX>(v);
     }
 }
 
@@ -176,7 +196,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const TX* __restrict__ x,
         float acc = 0.f;
         for (int k = 0; k < top; ++k) {
             const int e = idx[static_cast<int64_t>(t) * top + k];
-            const float wk = weight[static_cast<int64_t>(t) * top + k];
+            const float wk = weight ? weight[static_cast<int64_t>(t) * top + k] : 1.f;
             if (e >= experts) {
                 acc = fmaf(wk, to_f32<TX>(x[static_cast<int64_t>(t) * hidden + c]), acc);
                 continue;
@@ -194,20 +214,24 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const TX* __restrict__ x,
 }  // namespace
 
 extern "C" int pulse_moe_route(const float* z, const void* correction, int c_dtype, int* idx, float* weight, int tokens,
-                               int n, int top, hipStream_t stream) {
+                               int n, int top, int score_fn, int renorm, hipStream_t stream) {
+    PULSE_REQUIRE(score_fn == 0 || score_fn == 1, "moe_route: unknown score function %d", score_fn);
     PULSE_REQUIRE(tokens >= 0 && n > 0 && top > 0 && top <= n && z && idx && weight, "moe_route: bad arguments");
     PULSE_REQUIRE(n <= PULSE_WAVE * ROUTE_PER_LANE && top <= PULSE_WAVE,
                   "moe_route: at most %d router outputs and %d choices", PULSE_WAVE * ROUTE_PER_LANE, PULSE_WAVE);
     PULSE_REQUIRE(pulse_dtype_ok(c_dtype), "moe_route: bad dtype tag");
     if (tokens == 0) return 0;
     PULSE_DISPATCH_DTYPE(c_dtype, TW, hipLaunchKernelGGL(moe_route_kernel<TW>, dim3(tokens), dim3(64), 0, stream, z,
-                                                         static_cast<const TW*>(correction), idx, weight, n, top));
+                                                         static_cast<const TW*>(correction), idx, weight, n, top,
+                                                         score_fn, renorm));
     PULSE_LAUNCH_CHECK("moe_route");
     return 0;
 }
 
 extern "C" int pulse_moe_router(const void* x, int x_dtype, const void* w, const void* correction, int w_dtype, int* idx,
-                                float* weight, int tokens, int hidden, int n, int top, hipStream_t stream) {
+                                float* weight, int tokens, int hidden, int n, int top, int score_fn, int renorm,
+                                hipStream_t stream) {
+    PULSE_REQUIRE(score_fn == 0 || score_fn == 1, "moe_router: unknown score function %d", score_fn);
     PULSE_REQUIRE(tokens >= 0 && hidden > 0 && n > 0 && top > 0 && top <= n && x && w && idx && weight,
                   "moe_router: bad arguments");
     PULSE_REQUIRE(n <= PULSE_WAVE * ROUTE_PER_LANE && top <= PULSE_WAVE,
@@ -219,13 +243,16 @@ extern "C" int pulse_moe_router(const void* x, int x_dtype, const void* w, const
     PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(w_dtype, TW,
         hipLaunchKernelGGL((moe_router_kernel<TX, TW>), dim3(tokens), dim3(tokens <= 256 ? 1024 : 256), lds, stream,
                            static_cast<const TX*>(x),
-                           static_cast<const TW*>(w), static_cast<const TW*>(correction), idx, weight, hidden, n, top)));
+                           static_cast<const TW*>(w), static_cast<const TW*>(correction), idx, weight, hidden, n, top,
+                           score_fn, renorm)));
     PULSE_LAUNCH_CHECK("moe_router");
     return 0;
 }
 
 extern "C" int pulse_moe_gate_up(const void* x, int x_dtype, const void* wg, const void* wu, int w_dtype, const int* idx,
-                                 void* act, int tokens, int hidden, int ff, int experts, int top, hipStream_t stream) {
+                                 void* act, int tokens, int hidden, int ff, int experts, int top, const float* in_weight,
+                                 int act_kind, float limit, hipStream_t stream) {
+    PULSE_REQUIRE(act_kind == 0 || act_kind == 1, "moe_gate_up: unknown activation %d", act_kind);
     PULSE_REQUIRE(tokens >= 0 && hidden > 0 && ff > 0 && experts >= 0 && top > 0 && x && idx && act,
                   "moe_gate_up: bad arguments");
     PULSE_REQUIRE(experts == 0 || (wg && wu), "moe_gate_up: the experts' weights are missing");
@@ -236,7 +263,8 @@ extern "C" int pulse_moe_gate_up(const void* x, int x_dtype, const void* wg, con
     PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(w_dtype, TW,
         hipLaunchKernelGGL((moe_gate_up_kernel<TX, TW>), dim3(tokens * top, (ff + 63) / 64), dim3(256),
                            sizeof(float) * hidden, stream, static_cast<const TX*>(x), static_cast<const TW*>(wg),
-                           static_cast<const TW*>(wu), idx, static_cast<TX*>(act), hidden, ff, experts, top)));
+                           static_cast<const TW*>(wu), idx, static_cast<TX*>(act), hidden, ff, experts, top, in_weight,
+                           act_kind, limit)));
     PULSE_LAUNCH_CHECK("moe_gate_up");
     return 0;
 }
@@ -244,7 +272,7 @@ extern "C" int pulse_moe_gate_up(const void* x, int x_dtype, const void* wg, con
 extern "C" int pulse_moe_down(const void* x, const void* act, int x_dtype, const void* wd, int w_dtype, const int* idx,
                               const float* weight, float* out, int tokens, int hidden, int ff, int experts, int top,
                               hipStream_t stream) {
-    PULSE_REQUIRE(tokens >= 0 && hidden > 0 && ff > 0 && experts >= 0 && top > 0 && x && act && idx && weight && out,
+    PULSE_REQUIRE(tokens >= 0 && hidden > 0 && ff > 0 && experts >= 0 && top > 0 && x && act && idx && out,
                   "moe_down: bad arguments");
     PULSE_REQUIRE(experts == 0 || wd, "moe_down: the experts' weights are missing");
     PULSE_REQUIRE(pulse_dtype_ok(x_dtype) && pulse_dtype_ok(w_dtype), "moe_down: bad dtype tag");

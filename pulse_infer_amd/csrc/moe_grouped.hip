@@ -189,7 +189,9 @@ __global__ __launch_bounds__(256) void moe_gate_up_grouped_kernel(const bf16_t* 
                                                                   const int* __restrict__ tile_row0,
                                                                   const int* __restrict__ tile_rows,
                                                                   const int* __restrict__ num_tiles,
-                                                                  bf16_t* __restrict__ act, int hidden, int ff, int top) {
+                                                                  bf16_t* __restrict__ act, int hidden, int ff, int top,
+                                                                  const float* __restrict__ in_weight, int act_kind,
+                                                                  float limit) {
     const int tile = blockIdx.x;
     if (tile >= *num_tiles) return;
     const int e = tile_expert[tile], row0 = tile_row0[tile], rows = tile_rows[tile];
@@ -231,11 +233,19 @@ __global__ __launch_bounds__(256) void moe_gate_up_grouped_kernel(const bf16_t* 
     for (int rb = 0; rb < RB; ++rb) {
         if (pair[rb] < 0) continue;
         bf16_t* dst = act + static_cast<int64_t>(pair[rb]) * ff;
+        // an expert that is fed weight * x: both products are linear, so the factor goes onto their results
+        const float wgt = in_weight ? in_weight[pair[rb]] : 1.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             if (j0 + i < ff) {
-                const float g = acc[0][rb][i];
-                dst[j0 + i] = f32_to_bf16(g / (1.0f + expf(-g)) * acc[1][rb][i]);
+                float g = acc[0][rb][i] * wgt, u = acc[1][rb][i] * wgt;
+                if (act_kind == 1) {   // clamped: min(g, limit) * sigmoid(1.702 g) * (clamp(u) + 1)
+                    g = fminf(g, limit);
+                    u = fminf(fmaxf(u, -limit), limit);
+                    dst[j0 + i] = f32_to_bf16(g / (1.0f + expf(-1.702f * g)) * (u + 1.0f));
+                } else {
+                    dst[j0 + i] = f32_to_bf16(g / (1.0f + expf(-g)) * u);
+                }
             }
         }
     }
@@ -303,7 +313,7 @@ __global__ void moe_combine_kernel(const TX* __restrict__ x, const float* __rest
     float acc = 0.f;
     for (int k = 0; k < top; ++k) {
         const int e = idx[t * top + k];
-        const float w = weight[t * top + k];
+        const float w = weight ? weight[t * top + k] : 1.f;
         if (e >= experts) acc = fmaf(w, to_f32<TX>(x[at]), acc);
         else if (e >= 0) acc = fmaf(w, y[(t * top + k) * hidden + c], acc);
     }
@@ -332,7 +342,9 @@ static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 1
 extern "C" int pulse_moe_gate_up_grouped(const void* x, const void* wg, const void* wu, const int* order,
                                          const int* tile_expert, const int* tile_row0, const int* tile_rows,
                                          const int* num_tiles, int max_tiles, int tile_rows_max, void* act, int hidden,
-                                         int ff, int top, hipStream_t stream) {
+                                         int ff, int top, const float* in_weight, int act_kind, float limit,
+                                         hipStream_t stream) {
+    PULSE_REQUIRE(act_kind == 0 || act_kind == 1, "moe_gate_up_grouped: unknown activation %d", act_kind);
     PULSE_REQUIRE(hidden > 0 && ff > 0 && top > 0 && max_tiles > 0, "moe_gate_up_grouped: bad sizes");
     PULSE_REQUIRE(hidden % 8 == 0 && aligned16(x) && aligned16(wg) && aligned16(wu),
                   "moe_gate_up_grouped: rows must be multiples of 8 values and 16-byte aligned");
@@ -344,11 +356,11 @@ extern "C" int pulse_moe_gate_up_grouped(const void* x, const void* wg, const vo
     if (tile_rows_max == 32)
         hipLaunchKernelGGL(moe_gate_up_grouped_kernel<2>, dim3(max_tiles, (ff + 15) / 16), dim3(256), 0, stream, static_cast<const bf16_t*>(x),
                            static_cast<const bf16_t*>(wg), static_cast<const bf16_t*>(wu), order, tile_expert, tile_row0,
-                           tile_rows, num_tiles, static_cast<bf16_t*>(act), hidden, ff, top);
+                           tile_rows, num_tiles, static_cast<bf16_t*>(act), hidden, ff, top, in_weight, act_kind, limit);
     else
         hipLaunchKernelGGL(moe_gate_up_grouped_kernel<8>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(x),
                            static_cast<const bf16_t*>(wg), static_cast<const bf16_t*>(wu), order, tile_expert, tile_row0,
-                           tile_rows, num_tiles, static_cast<bf16_t*>(act), hidden, ff, top);
+                           tile_rows, num_tiles, static_cast<bf16_t*>(act), hidden, ff, top, in_weight, act_kind, limit);
     PULSE_LAUNCH_CHECK("moe_gate_up_grouped");
     return 0;
 }
@@ -376,7 +388,7 @@ extern "C" int pulse_moe_down_grouped(const void* act, const void* wd, const int
 
 extern "C" int pulse_moe_combine(const void* x, int x_dtype, const float* y, const int* idx, const float* weight,
                                  float* out, int tokens, int hidden, int experts, int top, hipStream_t stream) {
-    PULSE_REQUIRE(tokens >= 0 && hidden > 0 && top > 0 && x && y && idx && weight && out && pulse_dtype_ok(x_dtype),
+    PULSE_REQUIRE(tokens >= 0 && hidden > 0 && top > 0 && x && y && idx && out && pulse_dtype_ok(x_dtype),
                   "moe_combine: bad arguments");
     const int64_t total = static_cast<int64_t>(tokens) * hidden;
     if (total == 0) return 0;

@@ -6,6 +6,8 @@
 //   q += bq, k += bk, v += bv                                  (biases optional)
 //   q <- q / sqrt(mean over all nq*d values of q^2 + eps) * wq  (one norm over the row; wq [nq*d]; optional)
 //   k likewise with wk [nkv*d]
+//   or (norm 2) every head of q and of k divided by the root mean square of its own d values, without weights;
+//   a rotation keeps a head's sum of squares, so this is the same before or after it
 //   q, k <- rotated at the token's position on the first rotary_dim channels of every head
 //           (pairing 0: channels 2i, 2i+1; pairing 1: channels i, i + rotary_dim/2)
 //   v <- v * value_scale
@@ -24,7 +26,7 @@ namespace {
 struct PrepArgs {
     int nq, nkv, d, dv, D;
     int64_t x_stride, q_stride;
-    int norm;           // 0: none, 1: over the whole projection
+    int norm;           // 0: none, 1: over the whole projection, 2: every head by itself, no weights
     float eps;
     int rotary_dim, pairing;
     int page_size, num_pages, bt_width;
@@ -65,9 +67,21 @@ __global__ __launch_bounds__(256) void qkv_rows_kernel(const TX* __restrict__ x,
         }
     }
     float inv_q = 1.f, inv_k = 1.f;
+    float* inv_s = row_s + nqd + nkd;   // [nq + nkv], norm 2 only
     if (a.norm == 1) {
         inv_q = 1.0f / sqrtf(block_sum(sq, scratch) / static_cast<float>(nqd) + a.eps);
         if (a.write_kv) inv_k = 1.0f / sqrtf(block_sum(sk, scratch) / static_cast<float>(nkd) + a.eps);
+    } else if (a.norm == 2) {
+        __syncthreads();
+        const int lane = tid % PULSE_WAVE, wave = tid / PULSE_WAVE, waves = blockDim.x / PULSE_WAVE;
+        const int heads = a.nq + (a.write_kv ? a.nkv : 0);
+        for (int hh = wave; hh < heads; hh += waves) {
+            float ss = 0.f;
+            for (int c = lane; c < a.d; c += PULSE_WAVE) ss = fmaf(row_s[hh * a.d + c], row_s[hh * a.d + c], ss);
+            ss = wave_sum(ss);
+            if (lane == 0) inv_s[hh] = 1.0f / sqrtf(ss / static_cast<float>(a.d) + a.eps);
+        }
+        __syncthreads();
     } else {
         __syncthreads();
     }
@@ -77,6 +91,7 @@ __global__ __launch_bounds__(256) void qkv_rows_kernel(const TX* __restrict__ x,
     // a value of q or k, normed and rotated: element c of head hd of the vector that starts at row_s + base
     auto prepared = [&](int base, int hd, int c, float inv, const TW* w) -> float {
         const int at = base + hd * a.d + c;
+        if (a.norm == 2) inv = inv_s[base / a.d + hd];
         float u = row_s[at] * inv;
         if (w) u *= to_f32<TW>(w[at - base]);
         if (cs && c < a.rotary_dim) {
@@ -158,7 +173,8 @@ extern "C" int pulse_qkv_rows(const void* x, int x_dtype, int64_t x_stride, cons
     PULSE_REQUIRE(tokens >= 0 && nq > 0 && nkv > 0 && d > 0 && dv > 0, "qkv_rows: bad sizes");
     PULSE_REQUIRE(D >= d && D >= dv, "qkv_rows: the stored head width %d is below %d or %d", D, d, dv);
     PULSE_REQUIRE(pulse_dtype_ok(x_dtype) && pulse_dtype_ok(w_dtype) && pulse_dtype_ok(c_dtype), "qkv_rows: bad dtype tag");
-    PULSE_REQUIRE(norm == 0 || norm == 1, "qkv_rows: unknown norm %d", norm);
+    PULSE_REQUIRE(norm == 0 || norm == 1 || norm == 2, "qkv_rows: unknown norm %d", norm);
+    PULSE_REQUIRE(norm != 2 || (!wq && !wk), "qkv_rows: the norm of every head by itself has no weights");
     PULSE_REQUIRE(x && q_out && positions && token_entry, "qkv_rows: null pointer");
     PULSE_REQUIRE(!write_kv || (kcache && vcache && block_table && page_size > 0 && num_pages > 0 && bt_width > 0),
                   "qkv_rows: the cache is missing");
@@ -167,7 +183,7 @@ extern "C" int pulse_qkv_rows(const void* x, int x_dtype, int64_t x_stride, cons
     PULSE_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "qkv_rows: cos and sin come together");
     PULSE_REQUIRE(!cos_t || (rotary_dim > 0 && rotary_dim % 2 == 0 && rotary_dim <= d && (pairing == 0 || pairing == 1)),
                   "qkv_rows: bad rotation (dims %d of %d, pairing %d)", rotary_dim, d, pairing);
-    const size_t lds = sizeof(float) * (static_cast<size_t>(nq) * d + static_cast<size_t>(nkv) * d);
+    const size_t lds = sizeof(float) * (static_cast<size_t>(nq) * d + static_cast<size_t>(nkv) * d + nq + nkv);
     PULSE_REQUIRE(lds <= 60 * 1024, "qkv_rows: a token's q and k (%zu bytes in float32) do not fit the workgroup's memory", lds);
     if (tokens == 0) return 0;
     const int parts = tokens >= 512 ? 1 : min(16, (nq * D + 511) / 512);

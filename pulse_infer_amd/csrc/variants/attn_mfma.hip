@@ -115,6 +115,14 @@ struct MfmaArgs {
     // is stored (an output gate whose logits another product left); null: no gate.
     const bf16_t* gate;
     int64_t gate_stride;
+    int gate_width;        // 0: one gate logit a head; > 0: one for each of the first gate_width channels of a head
+                           // (gate[t * gate_stride + h * gate_width + channel]); channels beyond are stored ungated
+    // A sink: exp(sink[h]) is one more term of head h's softmax denominator, without key or value; null: none.
+    const float* sink;
+    // A cap on the scores: s * scale becomes cap * tanh(s * scale / cap).  The kernels keep raw scores s and multiply
+    // by scale * log2 e later, so the raw score becomes cap_out * tanh(s * cap_in) with cap_in = scale / cap and
+    // cap_out = cap / scale; cap_out 0: no cap.
+    float cap_in, cap_out;
 };
 
 // What the C entry points take besides their long lists (null: none of it).
@@ -125,12 +133,38 @@ struct PulseAttnExtras {
     int v_head0;           // < 0: nq + nkv
     float temp_coef;
     int temp_every;
+    const void* sink;      // float32 [nq], or null (not taken by pulse_attn_decode)
+    float softcap;         // 0: none (not taken by pulse_attn_decode)
+    int gate_width;        // see MfmaArgs
 };
 
-// 1 / l of a column and its head's gate in one factor.
-__device__ __forceinline__ float gated(float inv, const bf16_t* gate, int64_t gate_stride, int64_t row, int head) {
-    if (!gate) return inv;
+// 1 / l of a column and its head's gate in one factor (a gate a channel is applied channel by channel instead).
+__device__ __forceinline__ float gated(float inv, const bf16_t* gate, int64_t gate_stride, int64_t row, int head,
+                                       int gate_width = 0) {
+    if (!gate || gate_width > 0) return inv;
     return inv / (1.0f + expf(-bf16_to_f32(gate[row * gate_stride + head])));
+}
+
+// The factor of channel `ch` of a head under a gate a channel (1 without one).
+__device__ __forceinline__ float channel_gate(const bf16_t* gate, int64_t gate_stride, int gate_width, int64_t row,
+                                              int head, int ch) {
+    if (!gate || gate_width <= 0 || ch >= gate_width) return 1.f;
+    return 1.0f / (1.0f + expf(-bf16_to_f32(gate[row * gate_stride + static_cast<int64_t>(head) * gate_width + ch])));
+}
+
+// The sum of a column's weights with its head's sink in it; `m_log2` is the reference point of the weights'
+// exponents in units of log2 (weights are exp2(score * log2 e - m_log2)).
+__device__ __forceinline__ float with_sink(float l, float m_log2, const float* sink, int head) {
+    if (!sink) return l;
+    if (m_log2 == -INFINITY) return 1.f;
+    return l + exp2f(fminf(sink[head] * 1.4426950408889634f - m_log2, 126.f));
+}
+
+// A raw score under the cap (see MfmaArgs): tanh(x) = 1 - 2 / (exp(2x) + 1).
+__device__ __forceinline__ float capped(float s, float cap_in, float cap_out) {
+    if (cap_out == 0.f) return s;
+    const float e = __expf(2.f * s * cap_in);
+    return cap_out * (1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f));
 }
 
 // The split size for a step whose longest context is `live` (at most n_splits * split_size, what the launch was made
@@ -512,7 +546,7 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int j = j0 + 16 * t + 4 * kg + i;
-                float v = s[t][i] * a.scale_log2e;
+                float v = capped(s[t][i], a.cap_in, a.cap_out) * a.scale_log2e;
                 const bool seen = !needs_mask || (j <= pos_c && j >= lo_c && j >= split_begin && j < split_end);
                 v = (seen && col_ok) ? v : -INFINITY;
                 p[t][i] = v;
@@ -636,13 +670,14 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     const int64_t row = row0 + tc2;
     const int head = g * a.group + hc2;
     if (a.n_splits == 1 || (a.plan && hi < split_size)) {   // the only split of its item: nothing to merge
-        const float inv = gated(ll > 0.f ? 1.0f / ll : 0.f, a.gate, a.gate_stride, row, head);
+        ll = with_sink(ll, mm, a.sink, head);
+        const float inv = gated(ll > 0.f ? 1.0f / ll : 0.f, a.gate, a.gate_stride, row, head, a.gate_width);
         bf16_t* dst = a.out + row * a.o_stride + static_cast<int64_t>(head) * D;
         for (int ch = dd; ch < D; ch += 16) {
             float v = 0.f;
 #pragma unroll
             for (int w = 0; w < WAVES; ++w) v += wgt[w] * s_o[w][ch][c];
-            dst[ch] = f32_to_bf16(v * inv);
+            dst[ch] = f32_to_bf16(v * inv * channel_gate(a.gate, a.gate_stride, a.gate_width, row, head, ch));
         }
     } else {
         const int64_t slot = (row * a.nq + head) * a.n_splits + split;
@@ -812,7 +847,7 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float v = s[t][i];
+                float v = capped(s[t][i], a.cap_in, a.cap_out);
                 if (!inner) {
                     const int j = j0 + 16 * t + 4 * kg + i;
                     v = (col_ok && j <= pos_c && j >= lo_c) ? v : -INFINITY;
@@ -893,10 +928,16 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     l_part += __shfl_xor(l_part, 16, PULSE_WAVE);
     l_part += __shfl_xor(l_part, 32, PULSE_WAVE);
     if (col_ok) {
-        const float inv = gated(l_part > 0.f ? 1.0f / l_part : 0.f, a.gate, a.gate_stride, col_row, col_head);
+        l_part = with_sink(l_part, m == -INFINITY ? -INFINITY : m * c2, a.sink, col_head);
+        const float inv = gated(l_part > 0.f ? 1.0f / l_part : 0.f, a.gate, a.gate_stride, col_row, col_head, a.gate_width);
         bf16_t* dst = a.out + static_cast<int64_t>(col_row) * a.o_stride + static_cast<int64_t>(col_head) * D;
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) {
+            if (a.gate_width > 0) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[dt][i] *= channel_gate(a.gate, a.gate_stride, a.gate_width, col_row, col_head, dt * 16 + 4 * kg + i);
+            }
             const uint32_t w0 = static_cast<uint32_t>(f32_to_bf16(acc[dt][0] * inv)) |
                                 (static_cast<uint32_t>(f32_to_bf16(acc[dt][1] * inv)) << 16);
             const uint32_t w1 = static_cast<uint32_t>(f32_to_bf16(acc[dt][2] * inv)) |
@@ -1151,6 +1192,14 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
         for (int i = 0; i < AHEAD && i < V_STEPS; ++i) vw[i] = v_read(i);
         __builtin_amdgcn_sched_barrier(0);
         // the maximum is tracked on the raw scores (the scale is positive); p = exp2((s - m) * scale * log2 e)
+        if (a.cap_out != 0.f) {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int t = 0; t < KT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) s[ct][t][i] = capped(s[ct][t][i], a.cap_in, a.cap_out);
+        }
         bf16x8 pb[CT][KT / 2];
         bool moved = false;
         float alpha[CT];
@@ -1280,10 +1329,17 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
         l += __shfl_xor(l, 16, PULSE_WAVE);
         l += __shfl_xor(l, 32, PULSE_WAVE);
         if (col_ok[ct] && direct) {
-            const float inv = gated(l > 0.f ? 1.0f / l : 0.f, a.gate, a.gate_stride, col_row[ct], col_head);
+            l = with_sink(l, m[ct] == -INFINITY ? -INFINITY : m[ct] * c2, a.sink, col_head);
+            const float inv = gated(l > 0.f ? 1.0f / l : 0.f, a.gate, a.gate_stride, col_row[ct], col_head, a.gate_width);
             bf16_t* dst = a.out + static_cast<int64_t>(col_row[ct]) * a.o_stride + static_cast<int64_t>(col_head) * D;
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt) {
+                if (a.gate_width > 0) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        acc[ct][dt][i] *= channel_gate(a.gate, a.gate_stride, a.gate_width, col_row[ct], col_head,
+                                                       dt * 16 + 4 * kg + i);
+                }
                 const uint32_t w0 = static_cast<uint32_t>(f32_to_bf16(acc[ct][dt][0] * inv)) |
                                     (static_cast<uint32_t>(f32_to_bf16(acc[ct][dt][1] * inv)) << 16);
                 const uint32_t w1 = static_cast<uint32_t>(f32_to_bf16(acc[ct][dt][2] * inv)) |
@@ -1317,7 +1373,8 @@ __global__ __launch_bounds__(PR_THREADS) void attn_prefill_reduce_kernel(const f
                                                                         const int* __restrict__ items, int item_tokens,
                                                                         bf16_t* __restrict__ out, int64_t o_stride, int nq,
                                                                         int n_splits, int split_size,
-                                                                        const bf16_t* __restrict__ gate, int64_t gate_stride) {
+                                                                        const bf16_t* __restrict__ gate, int64_t gate_stride,
+                                                                        int gate_width, const float* __restrict__ sink) {
     const int item = blockIdx.x / item_tokens;
     const int tok = blockIdx.x % item_tokens;
     const int row0 = items[4 * item];
@@ -1341,7 +1398,12 @@ __global__ __launch_bounds__(PR_THREADS) void attn_prefill_reduce_kernel(const f
         // a split below the row's window holds sums of nothing (zeros), never stale memory: it was written
         acc += *reinterpret_cast<const f32x4*>(part_o + (base + z) * D + 4 * quad) * wz;
     }
-    const float inv = gated(ll > 0.f ? 1.0f / ll : 0.f, gate, gate_stride, row, head);
+    ll = with_sink(ll, mm, sink, head);
+    const float inv = gated(ll > 0.f ? 1.0f / ll : 0.f, gate, gate_stride, row, head, gate_width);
+    if (gate_width > 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] *= channel_gate(gate, gate_stride, gate_width, row, head, 4 * quad + i);
+    }
     const uint32_t w0 = static_cast<uint32_t>(f32_to_bf16(acc[0] * inv)) | (static_cast<uint32_t>(f32_to_bf16(acc[1] * inv)) << 16);
     const uint32_t w1 = static_cast<uint32_t>(f32_to_bf16(acc[2] * inv)) | (static_cast<uint32_t>(f32_to_bf16(acc[3] * inv)) << 16);
     *reinterpret_cast<u32x2*>(out + row * o_stride + static_cast<int64_t>(head) * D + 4 * quad) = u32x2{w0, w1};
@@ -1368,7 +1430,8 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
                                                                          int n_splits, int static_split_size, int hpw_log2,
                                                                          const int* __restrict__ live_context,
                                                                          const int* __restrict__ plan, int n_items,
-                                                                         const bf16_t* __restrict__ gate, int64_t gate_stride) {
+                                                                         const bf16_t* __restrict__ gate, int64_t gate_stride,
+                                                                         int gate_width, const float* __restrict__ sink) {
     __shared__ float s_w[MAX_SPLITS];      // hpw * n_splits <= MAX_SPLITS (hpw > 1 only with few splits)
     __shared__ float s_l[MAX_SPLITS];
     __shared__ f32x4 s_acc[REDUCE_GROUPS][REDUCE_QUADS];
@@ -1436,7 +1499,8 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
         for (int z = 0; z < valid; ++z) mm = fmaxf(mm, my_w[z]);
         float ll = 0.f;
         for (int z = 0; z < valid; ++z) ll += (my_w[z] == -INFINITY ? 0.f : exp2f(my_w[z] - mm)) * my_l[z];
-        inv = gated(ll > 0.f ? 1.0f / ll : 0.f, gate, gate_stride, row, head);
+        ll = with_sink(ll, mm, sink, head);
+        inv = gated(ll > 0.f ? 1.0f / ll : 0.f, gate, gate_stride, row, head, gate_width);
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < AHEAD; ++i) {
@@ -1456,7 +1520,8 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
         for (int gi = 1; gi < gph; ++gi) v += s_acc[grp + gi * hpw][quad];
         bf16_t* dst = out + row * o_stride + static_cast<int64_t>(head) * D + 4 * quad;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dst[e] = f32_to_bf16(v[e] * inv);
+        for (int e = 0; e < 4; ++e)
+            dst[e] = f32_to_bf16(v[e] * inv * channel_gate(gate, gate_stride, gate_width, row, head, 4 * quad + e));
     }
 }
 
@@ -1589,13 +1654,23 @@ struct Preparation {
 };
 
 // The gate of `ex` into the kernels' arguments, checked; the other extras are pulse_attn_decode's.
-int take_gate(MfmaArgs& a, const PulseAttnExtras* ex, int nq) {
-    a.gate = nullptr; a.gate_stride = 0;
+int take_gate(MfmaArgs& a, const PulseAttnExtras* ex, int nq, float scale = 0.f) {
+    a.gate = nullptr; a.gate_stride = 0; a.gate_width = 0;
+    a.sink = nullptr; a.cap_in = 0.f; a.cap_out = 0.f;
     a.plain_norm = 0; a.v_head0 = a.nq + a.nkv; a.temp_coef = 0.f; a.temp_every = 0;
-    if (!ex || !ex->gate) return 0;
-    PULSE_REQUIRE(ex->gate_stride >= nq, "attention: the gate's rows hold %lld values for %d heads",
+    if (!ex) return 0;
+    a.sink = static_cast<const float*>(ex->sink);
+    PULSE_REQUIRE(ex->softcap >= 0.f, "attention: a negative score cap");
+    if (ex->softcap > 0.f) {
+        PULSE_REQUIRE(scale > 0.f, "attention: a score cap needs a positive scale (and a kernel that takes one)");
+        a.cap_in = scale / ex->softcap; a.cap_out = ex->softcap / scale;
+    }
+    if (!ex->gate) return 0;
+    PULSE_REQUIRE(ex->gate_width >= 0 && ex->gate_width <= D, "attention: %d gated channels of a head of %d", ex->gate_width, D);
+    PULSE_REQUIRE(ex->gate_stride >= static_cast<int64_t>(nq) * (ex->gate_width > 0 ? ex->gate_width : 1),
+                  "attention: the gate's rows hold %lld values for %d heads",
                   static_cast<long long>(ex->gate_stride), nq);
-    a.gate = static_cast<const bf16_t*>(ex->gate); a.gate_stride = ex->gate_stride;
+    a.gate = static_cast<const bf16_t*>(ex->gate); a.gate_stride = ex->gate_stride; a.gate_width = ex->gate_width;
     return 0;
 }
 
@@ -1642,7 +1717,7 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
     a.plan = n_splits > 1 ? plan : nullptr;
     a.n_items = n_items;
     a.q_w = a.k_w = nullptr; a.cos_t = a.sin_t = nullptr; a.eps = 0.f; a.rotary_dim = 0; a.pairing = 0; a.new_key = 0;
-    if (take_gate(a, ex, nq)) return 1;
+    if (take_gate(a, ex, nq, scale)) return 1;
     if (prep && ex) {
         a.plain_norm = ex->plain_norm ? 1 : 0;
         a.v_head0 = ex->v_head0 >= 0 ? ex->v_head0 : nq + nkv;
@@ -1669,7 +1744,7 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
         while (hpw * 2 * n_splits <= REDUCE_GROUPS && hpw * 2 <= nq) { hpw *= 2; ++hpw_log2; }
         hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(n_items * per, (nq + hpw - 1) / hpw), dim3(REDUCE_THREADS), 0, stream,
                            part_o, part_ml, positions, items, per, a.out, o_stride, nq, n_splits, split_size, hpw_log2,
-                           a.live_context, a.plan, n_items, a.gate, a.gate_stride);
+                           a.live_context, a.plan, n_items, a.gate, a.gate_stride, a.gate_width, a.sink);
         PULSE_LAUNCH_CHECK("attn_mfma_reduce");
     }
     return 0;
@@ -1800,7 +1875,7 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
     a.live_context = nullptr;
     a.plan = nullptr;
     a.part_o = n_splits > 1 ? part_o : nullptr; a.part_ml = n_splits > 1 ? part_ml : nullptr;
-    if (take_gate(a, extras, nq)) return 1;
+    if (take_gate(a, extras, nq, scale)) return 1;
 #if PULSE_WIDE
     hipLaunchKernelGGL((attn_prefill_wide_kernel<WIDE_CT, 4, WIDE_NW>), dim3(n_items, nkv * a.head_chunks, n_splits),
                        dim3(WIDE_NW * PULSE_WAVE), 0, stream, a, 16 / gp);
@@ -1809,7 +1884,7 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
         const int item_tokens = WIDE_NW * WIDE_CT * (16 / gp);
         hipLaunchKernelGGL(attn_prefill_reduce_kernel, dim3(n_items * item_tokens, (nq + PR_HEADS - 1) / PR_HEADS),
                            dim3(PR_THREADS), 0, stream, part_o, part_ml, positions, items, item_tokens, a.out, o_stride, nq,
-                           n_splits, split_size, a.gate, a.gate_stride);
+                           n_splits, split_size, a.gate, a.gate_stride, a.gate_width, a.sink);
     }
 #else
     hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_items, nkv * a.head_chunks), dim3(WAVES * PULSE_WAVE), 0, stream, a,

@@ -94,7 +94,7 @@ class CausalLM:
     def forward(self, ctx: StepContext, cache_views: List[Any]) -> torch.Tensor:
         """Run the step's tokens through every run of the order; float32 logits [wanted, vocab]."""
         ws = ctx.workspace
-        h = ws.buffer("model.residual", ctx.num_tokens, self.hidden_size, torch.float32)
+        h = ws.buffer("model.residual", ctx.num_tokens, self.hidden_size * self.spec.streams, torch.float32)
         self.embedding.forward(ctx.token_ids, h)
         stream = ResidualStream(h)
         order = self.spec.order

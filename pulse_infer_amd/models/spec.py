@@ -81,10 +81,15 @@ class ModelSpec:
     final_norm_prefix: str = "model.norm"
     # position encodings by name; mixers refer to them through params["position"]
     positions: Dict[str, PartSpec] = field(default_factory=dict)
+    # rows of the residual a token (hyper-connections keep several streams); the embedding fills them all, blocks and
+    # the final norm must be of kinds that read that many
+    streams: int = 1
 
     def validate(self) -> None:
         if not self.layers:
             raise ValueError("a model needs at least one layer")
+        if self.streams < 1:
+            raise ValueError(f"a residual has at least one stream, got {self.streams}")
         for index, run in enumerate(self.order):
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"order[{index}] names layer {run.layer}, the model has {len(self.layers)}")

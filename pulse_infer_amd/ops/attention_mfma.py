@@ -23,25 +23,38 @@ def supported(head_dim: int, page_size: int, dtype: torch.dtype, cache_dtype: to
 class _Extras(ctypes.Structure):
     # as PulseAttnExtras of the kernel source
     _fields_ = [("gate", ctypes.c_void_p), ("gate_stride", ctypes.c_int64), ("plain_norm", ctypes.c_int),
-                ("v_head0", ctypes.c_int), ("temp_coef", ctypes.c_float), ("temp_every", ctypes.c_int)]
+                ("v_head0", ctypes.c_int), ("temp_coef", ctypes.c_float), ("temp_every", ctypes.c_int),
+                ("sink", ctypes.c_void_p), ("softcap", ctypes.c_float), ("gate_width", ctypes.c_int)]
 
 
 def _extras(what: str, tokens: int, nq: int, gate: Optional[torch.Tensor] = None, plain_norm: bool = False,
-            v_head0: int = -1, q_temperature: Optional[Tuple[float, int]] = None):
+            v_head0: int = -1, q_temperature: Optional[Tuple[float, int]] = None, gate_width: int = 0,
+            sink: Optional[torch.Tensor] = None, softcap: float = 0.0):
     """What the entry points take besides their lists, or a null pointer when there is none of it.  ``gate``: bfloat16
     [tokens, nq] (rows may be strided), the logits of an output gate: head h of token t leaves the kernel multiplied
     by sigmoid(gate[t, h]).  The rest is for ``attn_decode``: a norm of q and k without weights, the head number at
     which the raw values start in a row of the projection output, and a query temperature (coef, every):
-    q *= 1 + coef * ln(floor((position + 1) / every) + 1)."""
-    if gate is None and not plain_norm and v_head0 < 0 and q_temperature is None:
+    q *= 1 + coef * ln(floor((position + 1) / every) + 1).  ``gate_width`` > 0: the gate holds a logit for each of the
+    first ``gate_width`` channels of every head ([tokens, nq * gate_width]).  ``sink`` float32 [nq]: exp(sink[h]) is one
+    more term of head h's softmax denominator; ``softcap`` > 0: scaled scores become cap * tanh(score / cap)."""
+    if gate is None and not plain_norm and v_head0 < 0 and q_temperature is None and sink is None and not softcap:
         return None
     ex = _Extras()
     if gate is not None:
         _gpu(what, gate)
+        cols = nq * max(1, gate_width)
         _need(gate.dtype == torch.bfloat16 and gate.dim() == 2 and gate.shape[0] == tokens
-              and gate.shape[1] >= nq and gate.stride(1) == 1,
-              f"{what}: the gate must be bfloat16 [{tokens}, {nq}] with contiguous rows")
-        ex.gate, ex.gate_stride = gate.data_ptr(), gate.stride(0) if tokens > 1 else max(nq, gate.shape[1])
+              and gate.shape[1] >= cols and gate.stride(1) == 1,
+              f"{what}: the gate must be bfloat16 [{tokens}, {cols}] with contiguous rows")
+        ex.gate, ex.gate_stride = gate.data_ptr(), gate.stride(0) if tokens > 1 else max(cols, gate.shape[1])
+        ex.gate_width = int(gate_width)
+    if sink is not None:
+        _gpu(what, sink)
+        _need(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == nq,
+              f"{what}: the sinks must be float32 [{nq}]")
+        ex.sink = sink.data_ptr()
+    _need(softcap >= 0.0, f"{what}: a score cap must not be negative")
+    ex.softcap = float(softcap)
     ex.plain_norm = 1 if plain_norm else 0
     ex.v_head0 = int(v_head0)
     if q_temperature is not None:
@@ -147,7 +160,8 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
               items: torch.Tensor, scale: float, window: int, split_size: int, n_splits: int, max_context: int,
               part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor],
               live_context: Optional[torch.Tensor] = None, plan: Optional[torch.Tensor] = None,
-              gate: Optional[torch.Tensor] = None) -> None:
+              gate: Optional[torch.Tensor] = None, gate_width: int = 0, sink: Optional[torch.Tensor] = None,
+              softcap: float = 0.0) -> None:
     """Attention of decoded tokens and short portions.  ``split_size`` x ``n_splits`` is what the launch is made for
     (contexts up to ``max_context``); ``live_context`` (one int32 on the device: the longest context among the step's
     entries as it is now) lets the kernel cut the keys that are there evenly into the same number of splits;
@@ -178,7 +192,7 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
             _ptr(vcache), _ptr(positions), _ptr(block_table), _i32(block_table.shape[1]),
             _ptr(items), _i32(n_items), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages), _f32(scale),
             _i32(window), _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml),
-            _ptr(live_context), _ptr(plan), _extras("attn_mfma", tokens, nq, gate), _stream())
+            _ptr(live_context), _ptr(plan), _extras("attn_mfma", tokens, nq, gate, gate_width=gate_width, sink=sink, softcap=softcap), _stream())
 
 
 PLAN_MIN_KEYS = 256      # no split of a plan is shorter (what a workgroup costs beside its walk, in keys walked)
@@ -296,7 +310,8 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, 
                  vcache: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
                  items: torch.Tensor, scale: float, window: int, split_size: int = 0, n_splits: int = 1,
                  part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
-                 gate: Optional[torch.Tensor] = None) -> None:
+                 gate: Optional[torch.Tensor] = None, gate_width: int = 0, sink: Optional[torch.Tensor] = None,
+                 softcap: float = 0.0) -> None:
     """Attention for prompt portions: items of up to portion_tokens(group, d) tokens, keys shared through LDS.
     With ``n_splits > 1`` the keys are walked in splits of ``split_size`` (a multiple of 64) by workgroups of their
     own and merged by a second kernel; ``part_o`` / ``part_ml`` are float32 scratch of tokens * nq * n_splits * d
@@ -328,7 +343,7 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, 
             _ptr(items), _i32(items.numel() // ITEM_INTS), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages),
             _f32(scale), _i32(window), _i32(split_size if n_splits > 1 else 0), _i32(n_splits),
             _ptr(part_o if n_splits > 1 else None), _ptr(part_ml if n_splits > 1 else None),
-            _extras("attn_prefill", tokens, nq, gate), _stream())
+            _extras("attn_prefill", tokens, nq, gate, gate_width=gate_width, sink=sink, softcap=softcap), _stream())
 
 
 def decode_takes(d: int, rotary_dim: int, pairing: int) -> bool:

@@ -8,7 +8,7 @@ result tensor is asked for, and nothing falls back to another implementation.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Any, Optional
 
 import torch
 
@@ -125,15 +125,20 @@ def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
          _stream())
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor, slab: int = 0) -> None:
-    """out[t, i] = silu(gate) * up; gate_up holds [gate | up] halves (slab 0) or alternating slabs of ``slab`` columns."""
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, slab: int = 0, activation: str = "silu") -> None:
+    """out[t, i] = act(gate) * up, act silu or the tanh form of gelu; gate_up holds [gate | up] halves (slab 0) or
+    alternating slabs of ``slab`` columns."""
+    _need(activation in GATE_ACTIVATIONS, f"swiglu: unknown activation '{activation}'")
     _gpu("swiglu", gate_up, out)
     tokens, two_i = gate_up.shape
     _need(two_i % 2 == 0 and tuple(out.shape) == (tokens, two_i // 2), "swiglu: out must be [T, I] for gate_up [T, 2I]")
     _need(gate_up.is_contiguous() and out.is_contiguous() and gate_up.dtype == out.dtype,
           "swiglu: contiguous tensors of one storage type are needed")
     call("pulse_swiglu", _ptr(gate_up), _ptr(out), _i32(_tag(out, "swiglu")), _i32(tokens), _i32(two_i // 2),
-         _i32(slab), _stream())
+         _i32(slab), _i32(GATE_ACTIVATIONS[activation]), _stream())
 
 
 def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos_out: torch.Tensor, sin_out: torch.Tensor) -> None:
@@ -456,8 +461,13 @@ def qk_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight: Optional[
 
 def attn_generic(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
                  vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
-                 scale: float, window: int = 0, gate: Optional[torch.Tensor] = None) -> None:
+                 scale: float, window: int = 0, gate: Optional[torch.Tensor] = None, gate_width: int = 0,
+                 sink: Optional[torch.Tensor] = None, softcap: float = 0.0) -> None:
     """Paged causal attention, one wavefront per (token, head), float32 arithmetic.
+
+    ``gate_width`` > 0: the gate holds a logit for each of the first ``gate_width`` channels of every head
+    ([T, nq * gate_width]) instead of one a head.  ``sink`` float32 [nq]: exp(sink[h]) is one more term of head h's
+    softmax denominator.  ``softcap`` > 0: scaled scores become cap * tanh(score / cap).
 
     ``q`` is [T, >= nq*d] (rows may be strided, e.g. the front of a fused qkv buffer); ``out`` is [T, nq*d].
     ``gate`` [T, nq] of q's storage type (rows may be strided): head h of token t is multiplied by sigmoid(gate[t, h]).
@@ -474,13 +484,20 @@ def attn_generic(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, 
           "attn_generic: block_table must be contiguous int32 [entries, width]")
     if gate is not None:
         _gpu("attn_generic", gate)
-        _need(gate.dtype == q.dtype and gate.dim() == 2 and gate.shape[0] == tokens and gate.shape[1] >= nq
-              and gate.stride(1) == 1, f"attn_generic: the gate must be [{tokens}, {nq}] of q's storage type")
-    gate_stride = 0 if gate is None else (gate.stride(0) if tokens > 1 else max(nq, gate.shape[1]))
+        _need(0 <= gate_width <= d, f"attn_generic: {gate_width} gated channels of a head of {d}")
+        _need(gate.dtype == q.dtype and gate.dim() == 2 and gate.shape[0] == tokens
+              and gate.shape[1] >= nq * max(1, gate_width) and gate.stride(1) == 1,
+              f"attn_generic: the gate must be [{tokens}, {nq * max(1, gate_width)}] of q's storage type")
+    if sink is not None:
+        _gpu("attn_generic", sink)
+        _need(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == nq,
+              f"attn_generic: the sinks must be float32 [{nq}]")
+    gate_stride = 0 if gate is None else (gate.stride(0) if tokens > 1 else max(nq * max(1, gate_width), gate.shape[1]))
     call("pulse_attn_generic", _ptr(q), _i64(q.stride(0)), _ptr(out), _i64(out.stride(0)), _i32(_tag(q, "attn_generic")),
          _ptr(kcache), _ptr(vcache), _i32(_tag(kcache, "attn_generic")), _ptr(positions), _ptr(token_entry),
          _ptr(block_table), _i32(block_table.shape[1]), _i32(tokens), _i32(nq), _i32(nkv), _i32(d), _i32(page_size),
-         _i32(pages), _f32(scale), _i32(window), _ptr(gate), _i64(gate_stride), _stream())
+         _i32(pages), _f32(scale), _i32(window), _ptr(gate), _i64(gate_stride),
+         _i32(gate_width if gate is not None else 0), _ptr(sink), _f32(softcap), _stream())
 
 
 def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.Tensor] = None,
@@ -657,9 +674,9 @@ def qkv_rows(qkv: torch.Tensor, q_out: torch.Tensor, nq: int, nkv: int, d: int, 
              sin: Optional[torch.Tensor], rotary_dim: int, pairing: int, kcache: Optional[torch.Tensor],
              vcache: Optional[torch.Tensor], positions: torch.Tensor, token_entry: torch.Tensor,
              block_table: Optional[torch.Tensor], write_kv: bool = True, value_scale: float = 1.0,
-             norm: bool = True) -> None:
-    """q, k, v of ``qkv`` [T, nq*d + nkv*d + nkv*dv] -> biased, q and k normed over the whole row (``norm``, with
-    ``norm_weights`` = (wq [nq*d], wk [nkv*d]) or None), rotated; q to ``q_out`` [T, nq*stored], k and v (times
+             norm: Any = True) -> None:
+    """q, k, v of ``qkv`` [T, nq*d + nkv*d + nkv*dv] -> biased, q and k normed over the whole row (``norm`` True, with
+    ``norm_weights`` = (wq [nq*d], wk [nkv*d]) or None) or head by head without weights (``norm`` "head"), rotated; q to ``q_out`` [T, nq*stored], k and v (times
     ``value_scale``) to their pages, every head filled with zeros up to ``stored`` channels."""
     _gpu("qkv_rows", qkv, q_out, cos, sin, kcache, vcache, positions, token_entry, block_table)
     tokens = qkv.shape[0]
@@ -697,7 +714,7 @@ def qkv_rows(qkv: torch.Tensor, q_out: torch.Tensor, nq: int, nkv: int, d: int, 
         width = block_table.shape[1]
         c_tag = _tag(kcache, "qkv_rows")
     call("pulse_qkv_rows", _ptr(qkv), _i32(_tag(qkv, "qkv_rows")), _i64(qkv.stride(0)), _ptr(ptrs[0]), _ptr(ptrs[1]),
-         _ptr(ptrs[2]), _ptr(ptrs[3]), _ptr(ptrs[4]), _i32(w_tag or 0), _i32(1 if norm else 0), _f32(eps), _ptr(cos),
+         _ptr(ptrs[2]), _ptr(ptrs[3]), _ptr(ptrs[4]), _i32(w_tag or 0), _i32(2 if norm == "head" else (1 if norm else 0)), _f32(eps), _ptr(cos),
          _ptr(sin), _i32(rotary_dim if cos is not None else 0), _i32(pairing), _ptr(q_out), _i64(q_out.stride(0)),
          _ptr(kcache if write_kv else None), _ptr(vcache if write_kv else None), _i32(c_tag), _ptr(positions),
          _ptr(token_entry), _ptr(block_table if write_kv else None), _i32(width), _i32(tokens), _i32(nq), _i32(nkv),
@@ -807,8 +824,12 @@ def gated_rmsnorm(o: torch.Tensor, weight: torch.Tensor, gate: Optional[torch.Te
 
 # ---------------------------------------------------------------------------
 # Routed feed-forward
+ROUTER_SCORES = {"softmax": 0, "sigmoid": 1}
+EXPERT_ACTIVATIONS = {"silu": 0, "clamped_swish": 1}
+
+
 def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, idx: torch.Tensor,
-              weight: torch.Tensor) -> None:
+              weight: torch.Tensor, score: str = "softmax", renormalize: bool = True) -> None:
     """Softmax over a row of router logits, the ``top`` outputs with the largest score + correction, and their scores
     divided by their sum: idx int32 [T, top], weight float32 [T, top]."""
     _gpu("moe_route", logits, correction, idx, weight)
@@ -820,12 +841,15 @@ def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int
           and weight.dtype == torch.float32 and weight.is_contiguous() and tuple(weight.shape) == (tokens, top),
           f"moe_route: idx int32 and weight float32 must be [{tokens}, {top}]")
     call("pulse_moe_route", _ptr(logits), _ptr(correction), _i32(_tag(correction, "moe_route") if correction is not None else 0),
-         _ptr(idx), _ptr(weight), _i32(tokens), _i32(n), _i32(top), _stream())
+         _ptr(idx), _ptr(weight), _i32(tokens), _i32(n), _i32(top), _i32(ROUTER_SCORES[score]),
+         _i32(1 if renormalize else 0), _stream())
 
 
 def moe_router(x: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor], top: int, idx: torch.Tensor,
-               weight: torch.Tensor) -> None:
-    """``moe_route`` of the logits x w_router^T, which are formed in float32 inside the kernel."""
+               weight: torch.Tensor, score: str = "softmax", renormalize: bool = True) -> None:
+    """``moe_route`` of the logits x w_router^T, which are formed in float32 inside the kernel.  ``score``: softmax
+    over all outputs or a sigmoid of each; ``renormalize`` False leaves the chosen scores as the weights."""
+    _need(score in ROUTER_SCORES, f"moe_router: unknown score function '{score}'")
     _gpu("moe_router", x, w_router, correction, idx, weight)
     tokens, hidden = x.shape
     n = w_router.shape[0]
@@ -839,11 +863,23 @@ def moe_router(x: torch.Tensor, w_router: torch.Tensor, correction: Optional[tor
           f"moe_router: idx int32 and weight float32 must be [{tokens}, {top}]")
     call("pulse_moe_router", _ptr(x), _i32(_tag(x, "moe_router")), _ptr(w_router), _ptr(correction),
          _i32(_tag(w_router, "moe_router")), _ptr(idx), _ptr(weight), _i32(tokens), _i32(hidden), _i32(n), _i32(top),
-         _stream())
+         _i32(ROUTER_SCORES[score]), _i32(1 if renormalize else 0), _stream())
 
 
-def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, idx: torch.Tensor, act: torch.Tensor) -> None:
-    """act[(t, k)] = silu(gate_e x_t) * (up_e x_t) for e = idx[t, k] < experts; rows of identity experts are left alone."""
+def _in_weight(what: str, in_weight: Optional[torch.Tensor], tokens: int, top: int) -> None:
+    if in_weight is not None:
+        _gpu(what, in_weight)
+        _need(in_weight.dtype == torch.float32 and in_weight.is_contiguous() and tuple(in_weight.shape) == (tokens, top),
+              f"{what}: the weights on the experts' inputs must be float32 [{tokens}, {top}]")
+
+
+def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, idx: torch.Tensor, act: torch.Tensor,
+                in_weight: Optional[torch.Tensor] = None, activation: str = "silu", limit: float = 0.0) -> None:
+    """act[(t, k)] = silu(gate_e x_t) * (up_e x_t) for e = idx[t, k] < experts; rows of identity experts are left alone.
+    ``in_weight`` [T, top]: the expert is fed in_weight[t, k] * x_t.  ``activation`` "clamped_swish": with
+    g = min(gate, limit) and u = clamp(up, -limit, limit), act = g * sigmoid(1.702 g) * (u + 1)."""
+    _need(activation in EXPERT_ACTIVATIONS, f"moe_gate_up: unknown activation '{activation}'")
+    _in_weight("moe_gate_up", in_weight, x.shape[0], idx.shape[1])
     _gpu("moe_gate_up", x, w_gate, w_up, idx, act)
     tokens, hidden = x.shape
     experts, ff, h2 = w_gate.shape
@@ -855,12 +891,13 @@ def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, idx: 
     _need(idx.dtype == torch.int32 and idx.is_contiguous() and idx.shape[0] == tokens, "moe_gate_up: idx must be int32 [T, top]")
     call("pulse_moe_gate_up", _ptr(x), _i32(_tag(x, "moe_gate_up")), _ptr(w_gate), _ptr(w_up),
          _i32(_tag(w_gate, "moe_gate_up")), _ptr(idx), _ptr(act), _i32(tokens), _i32(hidden), _i32(ff), _i32(experts),
-         _i32(top), _stream())
+         _i32(top), _ptr(in_weight), _i32(EXPERT_ACTIVATIONS[activation]), _f32(limit), _stream())
 
 
-def moe_down(x: torch.Tensor, act: torch.Tensor, w_down: torch.Tensor, idx: torch.Tensor, weight: torch.Tensor,
-             out: torch.Tensor) -> None:
-    """out[t] = sum_k weight[t, k] * (down_e act[(t, k)] if e = idx[t, k] < experts else x[t]), float32."""
+def moe_down(x: torch.Tensor, act: torch.Tensor, w_down: torch.Tensor, idx: torch.Tensor,
+             weight: Optional[torch.Tensor], out: torch.Tensor) -> None:
+    """out[t] = sum_k weight[t, k] * (down_e act[(t, k)] if e = idx[t, k] < experts else x[t]), float32; ``weight``
+    None: every weight is one."""
     _gpu("moe_down", x, act, w_down, idx, weight, out)
     tokens, hidden = x.shape
     experts, h2, ff = w_down.shape
@@ -869,7 +906,8 @@ def moe_down(x: torch.Tensor, act: torch.Tensor, w_down: torch.Tensor, idx: torc
     _need(x.is_contiguous() and act.is_contiguous() and act.dtype == x.dtype and tuple(act.shape) == (tokens * top, ff),
           f"moe_down: act must be [{tokens * top}, {ff}] of x's storage type")
     _need(idx.dtype == torch.int32 and idx.is_contiguous() and tuple(idx.shape) == (tokens, top)
-          and weight.dtype == torch.float32 and weight.is_contiguous() and tuple(weight.shape) == (tokens, top),
+          and (weight is None or (weight.dtype == torch.float32 and weight.is_contiguous()
+                                  and tuple(weight.shape) == (tokens, top))),
           "moe_down: idx int32 and weight float32 must be [T, top]")
     _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (tokens, hidden),
           f"moe_down: out must be float32 [{tokens}, {hidden}]")
@@ -894,10 +932,12 @@ def moe_max_tiles(pairs: int, experts: int, tile_rows: int) -> int:
 
 def moe_grouped(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, idx: torch.Tensor,
                 weight: torch.Tensor, act: torch.Tensor, y: torch.Tensor, out: torch.Tensor, scratch: torch.Tensor,
-                tile_rows: int) -> None:
+                tile_rows: int, weight_on_input: bool = False, activation: str = "silu", limit: float = 0.0) -> None:
     """out[t] = sum_k weight[t, k] * (expert idx[t, k] of x[t], or x[t] itself for an identity expert), the experts'
     products grouped by expert on the matrix cores.  ``act`` bfloat16 [T * top, ff] and ``y`` float32 [T * top, hidden]
-    are scratch; ``scratch`` int32 holds 2 * T * top + 3 * moe_max_tiles + 1 entries."""
+    are scratch; ``scratch`` int32 holds 2 * T * top + 3 * moe_max_tiles + 1 entries.  ``weight_on_input``: an expert is
+    fed weight * x and the results are added as they are; ``activation`` / ``limit`` as for ``moe_gate_up``."""
+    _need(activation in EXPERT_ACTIVATIONS, f"moe_grouped: unknown activation '{activation}'")
     _gpu("moe_grouped", x, w_gate, w_up, w_down, idx, weight, act, y, out, scratch)
     tokens, hidden = x.shape
     experts, ff, h2 = w_gate.shape
@@ -925,8 +965,148 @@ def moe_grouped(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_dow
     call("pulse_moe_group", _ptr(idx), _i32(pairs), _i32(experts), _i32(tile_rows), _i32(tiles), rank, order, t_expert,
          t_row0, t_rows, count, _stream())
     call("pulse_moe_gate_up_grouped", _ptr(x), _ptr(w_gate), _ptr(w_up), order, t_expert, t_row0, t_rows, count, _i32(tiles),
-         _i32(tile_rows), _ptr(act), _i32(hidden), _i32(ff), _i32(top), _stream())
+         _i32(tile_rows), _ptr(act), _i32(hidden), _i32(ff), _i32(top), _ptr(weight if weight_on_input else None),
+         _i32(EXPERT_ACTIVATIONS[activation]), _f32(limit), _stream())
     call("pulse_moe_down_grouped", _ptr(act), _ptr(w_down), order, t_expert, t_row0, t_rows, count, _i32(tiles),
          _i32(tile_rows), _ptr(y), _i32(hidden), _i32(ff), _stream())
-    call("pulse_moe_combine", _ptr(x), _i32(_tag(x, "moe_grouped")), _ptr(y), _ptr(idx), _ptr(weight), _ptr(out),
+    call("pulse_moe_combine", _ptr(x), _i32(_tag(x, "moe_grouped")), _ptr(y), _ptr(idx),
+         _ptr(None if weight_on_input else weight), _ptr(out),
          _i32(tokens), _i32(hidden), _i32(experts), _i32(top), _stream())
+
+
+# ---------------------------------------------------------------------------
+# A residual in several streams, and the layer norm that reads it
+NORM_KINDS = {"layernorm": 0, "rmsnorm": 1}
+
+
+def embed_streams(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, bad_id: torch.Tensor, streams: int,
+                  scale: float = 1.0) -> None:
+    """out[t, s] = float32(table[ids[t]]) * scale for every stream s; out float32 [T, streams * hidden]."""
+    _gpu("embed_streams", ids, table, out, bad_id)
+    tokens = ids.numel()
+    vocab, hidden = table.shape
+    _int_vec("embed_streams: ids", ids)
+    _need(streams >= 1 and table.is_contiguous() and out.is_contiguous() and out.dtype == torch.float32
+          and tuple(out.shape) == (tokens, streams * hidden),
+          f"embed_streams: out must be contiguous float32 [{tokens}, {streams * hidden}]")
+    _need(bad_id.dtype == torch.int32 and bad_id.numel() >= 1, "embed_streams: bad_id must be int32[1]")
+    call("pulse_embed_streams", _ptr(ids), _ptr(table), _i32(_tag(table, "embed_streams")), _ptr(out), _i32(tokens),
+         _i32(hidden), _i32(vocab), _i32(streams), _ptr(bad_id), _f32(scale), _stream())
+
+
+MAX_STREAMS = 16
+
+
+def streams_step(x: torch.Tensor, streams: int, update: Optional[tuple] = None, in_weight: Optional[torch.Tensor] = None,
+                 norm: Optional[tuple] = None, out: Optional[torch.Tensor] = None,
+                 rows: Optional[torch.Tensor] = None) -> None:
+    """One pass over a residual of ``streams`` rows a token, x float32 [T, streams * H].
+
+    ``update`` = (y [T, H], mix float32 [streams, streams] indexed [from, to], out_factors float32 [streams]):
+    x_t <- sum_s mix[s, t] x_s + out_factors[t] * y, all streams at once, written back.  ``norm`` = (kind, weight,
+    bias or None, eps) with ``out`` [rows, H]: u = sum_s in_weight[s] x_s (None: the plain sum) over the new streams,
+    normed (kind "layernorm" or "rmsnorm") and rounded once; ``rows`` gathers (without an update only)."""
+    _gpu("streams_step", x, in_weight, out, rows)
+    _need(1 <= streams <= MAX_STREAMS, f"streams_step: 1 to {MAX_STREAMS} streams, got {streams}")
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and x.shape[1] % streams == 0,
+          "streams_step: x must be contiguous float32 [T, streams * H]")
+    tokens, hidden = x.shape[0], x.shape[1] // streams
+    y = mix = out_w = None
+    if update is not None:
+        y, mix, out_w = update
+        _gpu("streams_step", y, mix, out_w)
+        _need(rows is None, "streams_step: an update runs over all rows")
+        _need(y.is_contiguous() and tuple(y.shape) == (tokens, hidden), f"streams_step: y must be [{tokens}, {hidden}]")
+        _need(mix.dtype == torch.float32 and mix.is_contiguous() and tuple(mix.shape) == (streams, streams)
+              and out_w.dtype == torch.float32 and out_w.is_contiguous() and out_w.numel() == streams,
+              "streams_step: mix float32 [streams, streams] and out_factors float32 [streams]")
+    if in_weight is not None:
+        _need(in_weight.dtype == torch.float32 and in_weight.is_contiguous() and in_weight.numel() == streams,
+              "streams_step: in_weight must be float32 [streams]")
+    n_rows = tokens
+    w = b = None
+    kind, eps = 0, 0.0
+    if norm is not None:
+        name, w, b, eps = norm
+        _gpu("streams_step", w, b)
+        _need(name in NORM_KINDS, f"streams_step: unknown norm '{name}'")
+        kind = NORM_KINDS[name]
+        _need(out is not None, "streams_step: a norm needs its output")
+        if rows is not None:
+            _int_vec("streams_step: rows", rows)
+            n_rows = rows.numel()
+        _need(w.numel() == hidden and w.is_contiguous() and (b is None or (b.numel() == hidden and b.is_contiguous()
+                                                                           and b.dtype == w.dtype)),
+              f"streams_step: weight and bias must hold {hidden} values of one storage type")
+        _need(out.is_contiguous() and tuple(out.shape) == (n_rows, hidden),
+              f"streams_step: out must be [{n_rows}, {hidden}], got {tuple(out.shape)}")
+        _need(hidden * 4 <= 60 * 1024, f"streams_step: rows of {hidden} values are too long")
+    else:
+        _need(update is not None and out is None, "streams_step: nothing to do")
+    call("pulse_streams_step", _ptr(x), _i32(tokens), _i32(streams), _i32(hidden), _ptr(y),
+         _i32(_tag(y, "streams_step") if y is not None else 0), _ptr(mix), _ptr(out_w), _ptr(in_weight), _ptr(rows),
+         _i32(n_rows), _ptr(w), _ptr(b), _i32(_tag(w, "streams_step") if w is not None else 0), _i32(kind), _f32(eps),
+         _ptr(out if norm is not None else None), _i32(_tag(out, "streams_step") if norm is not None else 0), _stream())
+
+
+# ---------------------------------------------------------------------------
+# Selective state-space mixer
+def causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                state: torch.Tensor, n_state: int, positions: torch.Tensor, token_entry: torch.Tensor,
+                entry_start: torch.Tensor, entry_first_row: torch.Tensor, entry_slot: torch.Tensor, entries: int) -> None:
+    """out[t, c] = silu(bias[c] + sum_j taps[c, j] * input at position p - (K - 1) + j), a convolution along each
+    request's tokens; ``x`` [T, >= C] (rows may be strided), ``taps`` [C, K], ``state`` float32 [slots, C, n_state +
+    K - 1], whose last K - 1 values a channel hold the inputs that came last and are moved on to this step's end."""
+    _gpu("causal_conv", x, taps, bias, out, state, positions, token_entry, entry_start, entry_first_row, entry_slot)
+    tokens = x.shape[0]
+    channels, k = taps.shape
+    _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[1] >= channels and out.dim() == 2 and out.stride(1) == 1
+          and tuple(out.shape) == (tokens, channels) and out.dtype == x.dtype,
+          f"causal_conv: x [T, >= {channels}] and out [T, {channels}] of one storage type with contiguous rows")
+    _need(taps.is_contiguous() and (bias is None or (bias.is_contiguous() and bias.numel() == channels
+                                                     and bias.dtype == taps.dtype)),
+          "causal_conv: taps [C, K] and bias [C] contiguous and of one storage type")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 3 and state.shape[1] == channels
+          and state.shape[2] == n_state + k - 1, f"causal_conv: state must be float32 [slots, {channels}, {n_state + k - 1}]")
+    _int_vec("causal_conv: positions", positions, tokens)
+    _int_vec("causal_conv: token_entry", token_entry, tokens)
+    _int_vec("causal_conv: entry_start", entry_start, entries)
+    _int_vec("causal_conv: entry_first_row", entry_first_row, entries + 1)
+    _int_vec("causal_conv: entry_slot", entry_slot, entries)
+    call("pulse_causal_conv", _ptr(x), _i64(x.stride(0) if tokens > 1 else x.shape[1]), _i32(_tag(x, "causal_conv")),
+         _ptr(taps), _ptr(bias), _i32(_tag(taps, "causal_conv")), _ptr(out), _i64(out.stride(0) if tokens > 1 else channels),
+         _ptr(state), _i32(state.shape[0]), _i32(n_state), _ptr(positions), _ptr(token_entry), _ptr(entry_start),
+         _ptr(entry_first_row), _ptr(entry_slot), _i32(tokens), _i32(entries), _i32(channels), _i32(k), _stream())
+
+
+def selective_scan(x: torch.Tensor, dt_raw: torch.Tensor, bc: torch.Tensor, b0: int, c0: int, z: Optional[torch.Tensor],
+                   y: torch.Tensor, dt_bias: Optional[torch.Tensor], a_log: torch.Tensor, d_skip: Optional[torch.Tensor],
+                   state: torch.Tensor, entry_start: torch.Tensor, entry_first_row: torch.Tensor,
+                   entry_slot: torch.Tensor, entries: int) -> None:
+    """The recurrence of a selective state-space mixer over every entry's tokens in order:
+    dt = softplus(dt_raw + dt_bias); S[c, n] <- exp(dt A[c, n]) S[c, n] + dt x_c B_n with A = -exp(a_log);
+    y_c = (sum_n S[c, n] C_n + d_skip_c x_c) * silu(z_c).  ``bc`` holds B at columns b0.. and C at c0.. of a row;
+    ``state`` float32 [slots, C, >= N]: its first N values a channel are S (zeros for an entry that starts at 0)."""
+    _gpu("selective_scan", x, dt_raw, bc, z, y, dt_bias, a_log, d_skip, state, entry_start, entry_first_row, entry_slot)
+    tokens = x.shape[0]
+    channels, n_state = a_log.shape
+    rows2 = lambda t: t.dim() == 2 and t.stride(1) == 1 and t.shape[0] == tokens and t.dtype == x.dtype
+    _need(rows2(x) and rows2(dt_raw) and rows2(bc) and rows2(y) and (z is None or rows2(z)),
+          "selective_scan: x, dt_raw, bc, z and y must be matrices of one storage type with contiguous rows")
+    _need(x.shape[1] >= channels and dt_raw.shape[1] >= channels and y.shape[1] >= channels
+          and (z is None or z.shape[1] >= channels), f"selective_scan: rows of at least {channels} channels")
+    _need(b0 >= 0 and c0 >= 0 and bc.shape[1] >= max(b0, c0) + n_state, "selective_scan: B and C lie outside their rows")
+    small = [t for t in (dt_bias, d_skip) if t is not None]
+    _need(a_log.is_contiguous() and all(t.is_contiguous() and t.numel() == channels and t.dtype == a_log.dtype for t in small),
+          "selective_scan: a_log [C, N], dt_bias [C] and d_skip [C] contiguous and of one storage type")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 3 and state.shape[1] == channels
+          and state.shape[2] >= n_state, f"selective_scan: state must be float32 [slots, {channels}, >= {n_state}]")
+    _int_vec("selective_scan: entry_start", entry_start, entries)
+    _int_vec("selective_scan: entry_first_row", entry_first_row, entries + 1)
+    _int_vec("selective_scan: entry_slot", entry_slot, entries)
+    stride = lambda t, cols: t.stride(0) if tokens > 1 else max(cols, t.shape[1])
+    call("pulse_selective_scan", _ptr(x), _i64(stride(x, channels)), _ptr(dt_raw), _i64(stride(dt_raw, channels)),
+         _ptr(bc), _i64(stride(bc, bc.shape[1])), _i32(b0), _i32(c0), _ptr(z), _i64(stride(z, channels) if z is not None else 0),
+         _ptr(y), _i64(stride(y, channels)), _i32(_tag(x, "selective_scan")), _ptr(dt_bias), _ptr(a_log), _ptr(d_skip),
+         _i32(_tag(a_log, "selective_scan")), _ptr(state), _i32(state.shape[0]), _i32(state.shape[2]), _ptr(entry_start),
+         _ptr(entry_first_row), _ptr(entry_slot), _i32(entries), _i32(channels), _i32(n_state), _stream())

@@ -22,6 +22,9 @@ Variations, all parameters of the part:
 * ``output_gate = True``: head h's output is multiplied by sigmoid(g_h), g = x Wg^T with Wg [heads, hidden] (one
   number a token and head), before the output projection; Wg's rows ride behind the other projections in the
   stacked weight, and the attention kernels apply the gate as they store their result;
+* ``score_cap = c``: a scaled score s becomes c * tanh(s / c) before the softmax;
+* ``sink = True``: a learned number per query head (tensor ``sink`` [heads]) whose exponential is one more term of
+  the softmax's denominator; it has no key and no value;
 * ``names``: the tensors' names below the part's prefix.
 """
 from __future__ import annotations
@@ -55,10 +58,12 @@ class PagedAttention(Part):
         if params.get("qk_norm", False) and params.get("qk_norm_weights", True):
             specs[names["q_norm"]] = TensorSpec((d,), kind="norm")
             specs[names["k_norm"]] = TensorSpec((d,), kind="norm")
+        if params.get("sink", False):
+            specs[names["sink"]] = TensorSpec((nq,), kind="linear", fan_in=4)
         return specs
 
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
-             "gate": "g_proj.weight", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
+             "gate": "g_proj.weight", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "sink": "sink"}
     GATE_PAD = 16   # the gate's rows of the stacked weight are filled up with zero rows to a multiple of this, so that
                     # the projection output's rows keep the alignment the kernels' 16-byte accesses need
 
@@ -107,6 +112,7 @@ class PagedAttention(Part):
             if self.q_temperature[1] <= 0:
                 raise ValueError(f"query_temperature.every must be positive, got {self.q_temperature[1]}")
         self.output_gate = bool(params.get("output_gate", False))
+        self._read_score_form(params)
         self.position = params.get("position")
         self.encodings = build.positions
         if self.position is not None and self.position not in self.encodings:
@@ -131,8 +137,23 @@ class PagedAttention(Part):
         weighted = self.qk_norm and not self.plain_norm
         self.q_w = load.get(names["q_norm"]) if weighted else None
         self.k_w = load.get(names["k_norm"]) if weighted else None
+        self.sink = self._load_sink(load, names["sink"]) if params.get("sink", False) else None
         self.act_dtype = build.act_dtype
         self.options = build.options
+
+    gate_width = 0     # > 0: the output gate has a logit for each of that many channels of a head (a subclass's)
+    score_cap = 0.0
+    sink = None
+
+    def _read_score_form(self, params: Dict[str, Any]) -> None:
+        self.score_cap = float(params.get("score_cap") or 0.0)
+        if self.score_cap < 0.0:
+            raise ValueError(f"a score cap must be positive, got {self.score_cap}")
+
+    @staticmethod
+    def _load_sink(load: Any, name: str) -> torch.Tensor:
+        """The sinks as float32 [heads], whatever the checkpoint's storage type."""
+        return load.get(name).to(torch.float32).contiguous()
 
     def cache_spec(self) -> PagedKVSpec:
         return PagedKVSpec(self.nkv, self.d, int(self.window) if self.window is not None else None)
@@ -188,6 +209,8 @@ class PagedAttention(Part):
         token, the matrix-core kernel takes the sizes, and norm weights and rotation are of the kinds it prepares."""
         if self.options.get("decode_from_raw", True) is False or not self.uses_matrix_cores(qkv, cache):
             return False
+        if self.score_cap or self.sink is not None:
+            return False
         if "static:attention.single_tokens" not in ctx.extras:
             ctx.extras["static:attention.single_tokens"] = all(e.count == 1 for e in ctx.entries)
         if not ctx.extras["static:attention.single_tokens"]:
@@ -207,7 +230,8 @@ class PagedAttention(Part):
         window = int(self.window) if self.window is not None else 0
         if not self.uses_matrix_cores(q, cache):
             kernels.attn_generic(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
-                                 ctx.token_entry, table, self.scale, window, gate=gate)
+                                 ctx.token_entry, table, self.scale, window, gate=gate, gate_width=self.gate_width,
+                                 sink=self.sink, softcap=self.score_cap)
             return
         group = self.nq // self.nkv
         per = attention_mfma.tokens_per_item(group)
@@ -234,7 +258,7 @@ class PagedAttention(Part):
                 part_ml = ctx.workspace.buffer("attention.portion_part_ml", rows, 2, torch.float32)
             attention_mfma.attn_prefill(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
                                         table, long_items, self.scale, window, split_size, n_splits, part_o, part_ml,
-                                        gate=gate)
+                                        gate=gate, gate_width=self.gate_width, sink=self.sink, softcap=self.score_cap)
         if short_items is not None:
             # a recorded step passes its context bucket as max_context: its splits must cover that
             max_context = ctx.max_context if long_items is None else short_context
@@ -276,4 +300,5 @@ class PagedAttention(Part):
             attention_mfma.attn_mfma(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
                                      table, short_items, self.scale, window, split_size, n_splits,
                                      max_context, part_o, part_ml,
-                                     live_context=ctx.live_context if plan is None else None, plan=plan, gate=gate)
+                                     live_context=ctx.live_context if plan is None else None, plan=plan, gate=gate,
+                                     gate_width=self.gate_width, sink=self.sink, softcap=self.score_cap)

@@ -4,8 +4,13 @@ of different widths.  Window, grouped key/value heads, rotation on the first cha
 those of ``attention``; so are the attention kernels, which this part inherits.
 
 Parameters beyond those of ``attention``: ``value_dim`` (default ``head_dim``); ``bias`` (q, k and v have biases,
-named by ``names`` as ``q_bias`` ...); ``qk_norm``: "projection" or False; ``qk_norm_eps``; ``out_scale`` (a factor on
-the result; it is multiplied into the values as they are stored, in float32 before their one rounding).
+named by ``names`` as ``q_bias`` ...); ``qk_norm``: "projection", "head" (every head of q and k divided by its own root
+mean square, no weights; the same before or after the rotation, which keeps a head's sum of squares) or False;
+``qk_norm_eps``; ``out_scale`` (a factor on the result; it is multiplied into the values as they are stored, in
+float32 before their one rounding); ``output_gate``: "channel": the heads' outputs are multiplied element by element
+by sigmoid(Wg x), Wg [heads * value_dim, hidden] (tensor ``gate``), whose rows ride behind q, k and v in the stacked
+projection and whose sigmoid the attention kernels apply as they store; ``score_cap`` and ``sink`` as for
+``attention``.
 
 Keys and values are stored with one width D = max(head_dim, value_dim) rounded up to a multiple of 16, the missing
 channels as zeros: zero key channels add nothing to a score, and zero value channels come out as zeros, which meet
@@ -34,7 +39,7 @@ def stored_width(d: int, dv: int) -> int:
 @MIXERS.register("attention_rows")
 class RowPreparedAttention(PagedAttention):
     NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "q_bias": "q.b", "k_bias": "k.b", "v_bias": "v.b",
-             "q_norm": "q.norm", "k_norm": "k.norm"}
+             "q_norm": "q.norm", "k_norm": "k.norm", "gate": "g", "sink": "sink"}
 
     @classmethod
     def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
@@ -51,9 +56,13 @@ class RowPreparedAttention(PagedAttention):
             specs[n["q_bias"]] = TensorSpec((nq * d,), fan_in=hidden)
             specs[n["k_bias"]] = TensorSpec((nkv * d,), fan_in=hidden)
             specs[n["v_bias"]] = TensorSpec((nkv * dv,), fan_in=hidden)
-        if params.get("qk_norm", False):
+        if params.get("qk_norm", False) == "projection":
             specs[n["q_norm"]] = TensorSpec((nq * d,), kind="norm")
             specs[n["k_norm"]] = TensorSpec((nkv * d,), kind="norm")
+        if params.get("output_gate", False):
+            specs[n["gate"]] = TensorSpec((nq * dv, hidden), fan_in=hidden)
+        if params.get("sink", False):
+            specs[n["sink"]] = TensorSpec((nq,), kind="linear", fan_in=4)
         return specs
 
     @classmethod
@@ -87,9 +96,15 @@ class RowPreparedAttention(PagedAttention):
         if self.window is not None and int(self.window) <= 0:
             raise ValueError(f"an attention window must be positive, got {self.window}")
         norm = params.get("qk_norm", False)
-        if norm not in (False, "projection"):
-            raise ValueError(f"attention_rows norms q and k over the 'projection' or not at all, got {norm!r}")
+        if norm not in (False, None, "projection", "head"):
+            raise ValueError(f"attention_rows norms q and k over the 'projection', by 'head' or not at all, got {norm!r}")
         self.row_norm = norm == "projection"
+        self.head_norm = norm == "head"
+        gate = params.get("output_gate", False)
+        if gate not in (False, None, "channel"):
+            raise ValueError(f"attention_rows has an output gate by 'channel' or none, got {gate!r}")
+        self.channel_gate = gate == "channel"
+        self._read_score_form(params)
         self.eps = float(params.get("qk_norm_eps", 0.0))
         self.out_scale = float(params.get("out_scale", 1.0))
         self.position = params.get("position")
@@ -99,7 +114,11 @@ class RowPreparedAttention(PagedAttention):
                            f"{sorted(self.encodings)}")
         load = build.loader
         n = {k: joined(prefix, v) for k, v in self.tensor_names(params).items()}
-        self.qkv = Linear(load.get_concat([n["q"], n["k"], n["v"]]), build.mode)
+        self.qkv = Linear(load.get_concat([n["q"], n["k"], n["v"]] + ([n["gate"]] if self.channel_gate else [])),
+                          build.mode)
+        self.kv_cols = self.nq * self.qk_dim + self.nkv * (self.qk_dim + self.v_dim)   # where the gate's columns start
+        self.gate_width = self.v_dim if self.channel_gate else 0
+        self.sink = self._load_sink(load, n["sink"]) if params.get("sink", False) else None
         self.biases = tuple(load.get(n[k]) for k in ("q_bias", "k_bias", "v_bias")) if params.get("bias", False) else None
         self.norm_weights = (load.get(n["q_norm"]), load.get(n["k_norm"])) if self.row_norm else None
         o = load.get(n["o"])
@@ -132,7 +151,7 @@ class RowPreparedAttention(PagedAttention):
         tokens = x.shape[0]
         ws = ctx.workspace
         write = cache.writable
-        rows = None if write else self.nq * self.qk_dim
+        rows = None if (write or self.channel_gate) else self.nq * self.qk_dim
         cols = self.qkv.out_features if rows is None else rows
         qkv = ws.buffer("attention_rows.qkv", tokens, cols, self.act_dtype)
         self.qkv.forward(x, qkv, rows=rows)
@@ -143,8 +162,10 @@ class RowPreparedAttention(PagedAttention):
                          self.eps, tables.cos if tables is not None else None,
                          tables.sin if tables is not None else None, tables.rotary_dim if tables is not None else 0,
                          tables.pairing if tables is not None else 0, cache.keys, cache.values, ctx.positions,
-                         ctx.token_entry, table, write_kv=write, value_scale=self.out_scale, norm=self.row_norm)
-        self.attend(q, out, ctx, cache, table)
+                         ctx.token_entry, table, write_kv=write, value_scale=self.out_scale,
+                         norm="head" if self.head_norm else self.row_norm)
+        gate = qkv[:, self.kv_cols:self.kv_cols + self.nq * self.v_dim] if self.channel_gate else None
+        self.attend(q, out, ctx, cache, table, gate=gate)
 
     def decodes_from_raw(self, ctx, cache, qkv, tables) -> bool:
         return False

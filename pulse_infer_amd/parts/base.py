@@ -219,6 +219,21 @@ class LazyNorm:
         return self.norm.apply(self.h, None, out)
 
 
+@dataclass
+class StreamUpdate:
+    """An update of a residual kept in several streams that has not been done yet: every stream becomes a mix of the
+    old ones plus a factor of its own times the sublayer's result ``y`` [T, H]: x_t <- sum_s mix[s, t] x_s +
+    out[t] * y.  A norm that says ``takes_streams`` does it inside its own kernel; anyone else calls ``apply_to``."""
+
+    y: torch.Tensor
+    mix: torch.Tensor     # float32 [streams, streams], indexed [from, to]
+    out: torch.Tensor     # float32 [streams]
+
+    def apply_to(self, h: torch.Tensor) -> None:
+        from ..ops import kernels
+        kernels.streams_step(h, self.out.numel(), update=(self.y, self.mix, self.out))
+
+
 class ResidualStream:
     """The float32 residual ``h`` and the update that has not been added to it yet.
 
@@ -241,6 +256,11 @@ class ResidualStream:
         pending, self.pending = self.pending, None
         if pending is not None:
             self.copy = None
+        if isinstance(pending, StreamUpdate):
+            if getattr(norm, "takes_streams", False):
+                return pending
+            pending.apply_to(self.h)
+            return None
         if pending is not None and pending.dim() == 3 and not getattr(norm, "takes_parts", False):
             from ..ops import kernels
             kernels.residual_add(self.h, pending)
@@ -263,7 +283,10 @@ class ResidualStream:
         lies in)."""
         if self.pending is not None:
             from ..ops import kernels
-            kernels.residual_add(self.h, self.pending)
+            if isinstance(self.pending, StreamUpdate):
+                self.pending.apply_to(self.h)
+            else:
+                kernels.residual_add(self.h, self.pending)
             self.pending = None
             self.copy = None
 
@@ -279,7 +302,10 @@ class ResidualStream:
             return
         if self.pending is not None:
             from ..ops import kernels
-            kernels.residual_add(self.h, self.pending)
+            if isinstance(self.pending, StreamUpdate):
+                self.pending.apply_to(self.h)
+            else:
+                kernels.residual_add(self.h, self.pending)
         self.pending = delta
 
 

@@ -11,6 +11,9 @@ h <- h + mixer(norm(h)).
 ``postnorm``: h <- norm_a(alpha h + ls_a * mixer(h)); h <- norm_b(alpha h + ls_b * ffn(h)): the
 sublayers read the stream itself, the norm comes after the sum, ``alpha`` weighs the
 stream in it and ``ls`` are optional factors, one a column, on a sublayer's result.
+
+``hyper``: the residual is S streams x_1 .. x_S.  Sublayer q reads u = sum_s in_q[s] x_s through its norm, and its
+result y goes back as x_t <- sum_s mix_q[s, t] x_s + out_q[t] * y, all streams at once from the old ones.
 """
 from __future__ import annotations
 
@@ -21,7 +24,8 @@ import torch
 from ..models.spec import LayerSpec
 from ..weights.store import TensorSpec
 from ..ops import kernels
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BuildContext, Part, ResidualStream, StepContext, joined, says
+from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BuildContext, Part, ResidualStream, StepContext, StreamUpdate,
+                   joined, says)
 
 
 @BLOCKS.register("prenorm")
@@ -264,3 +268,105 @@ class PostNormBlock(Part):
         self._close(stream, ctx, "mixer_norm", self.mixer.forward(self._rows(stream, ctx), ctx, cache))
         if self.ffn is not None:
             self._close(stream, ctx, "ffn_norm", self.ffn.forward(self._rows(stream, ctx), ctx))
+
+
+@BLOCKS.register("hyper")
+class HyperConnectionBlock(Part):
+    """A pre-norm layer around a residual of several streams (hyper-connections).
+
+    Block parameters: ``streams``; ``mixer_norm`` / ``ffn_norm``: the norms' tensor prefixes below the layer's;
+    ``mixer_hc`` / ``ffn_hc``: the prefixes of a sublayer's connection tensors, ``<prefix>.in`` [streams],
+    ``<prefix>.out`` [streams] and ``<prefix>.mix`` [streams, streams] (indexed [from, to]); ``learned`` False: there
+    are no such tensors, every factor is one and the streams do not mix (with one stream that is the plain residual
+    sum x <- x + sublayer(norm(x))).  The norms must say
+    ``takes_streams`` (they read the weighted sum of the streams and do a pending update on the way); a layer
+    without a feed-forward ends after the mixer.
+
+    The update of the streams is not a launch of its own: it is handed on as a ``StreamUpdate`` and done by the
+    kernel of the norm that reads the residual next (this layer's second norm, the next layer's first, the model's
+    last).  Connection tensors are kept in float32 whatever their storage type."""
+
+    NORM_PLACES = ("mixer_norm", "ffn_norm")
+    CONNECTIONS = (("mixer_norm", "mixer_hc"), ("ffn_norm", "ffn_hc"))
+
+    @classmethod
+    def _places(cls, layer: LayerSpec):
+        return [pair for pair in cls.CONNECTIONS if pair[0] == "mixer_norm" or layer.ffn is not None]
+
+    @classmethod
+    def layer_weight_specs(cls, layer: LayerSpec) -> Dict[str, TensorSpec]:
+        p = layer.block.params
+        streams = int(p["streams"])
+        out: Dict[str, TensorSpec] = {}
+        for which, hc in cls._places(layer):
+            norm = layer.norm(which)
+            for name, spec in NORMS.get(norm.kind).weight_specs(norm.params).items():
+                out[joined(joined(layer.prefix, p[which]), name)] = spec
+            if not p.get("learned", True):
+                continue
+            sub = joined(layer.prefix, p[hc])
+            out[joined(sub, "in")] = TensorSpec((streams,), kind="linear", fan_in=streams * streams)
+            out[joined(sub, "out")] = TensorSpec((streams,), kind="linear", fan_in=2)
+            out[joined(sub, "mix")] = TensorSpec((streams, streams), kind="linear", fan_in=streams)
+        parts = [(layer.mixer, MIXERS)] + ([(layer.ffn, FEED_FORWARDS)] if layer.ffn is not None else [])
+        for part, registry in parts:
+            sub = joined(layer.prefix, part.params.get("prefix", ""))
+            for name, spec in registry.get(part.kind).weight_specs(part.params).items():
+                out[joined(sub, name)] = spec
+        return out
+
+    def __init__(self, layer: LayerSpec, build: BuildContext):
+        p = layer.block.params
+        self.streams = int(p["streams"])
+        self.mixer = MIXERS.get(layer.mixer.kind)(layer.mixer.params,
+                                                  joined(layer.prefix, layer.mixer.params.get("prefix", "")), build)
+        self.ffn = None
+        if layer.ffn is not None:
+            self.ffn = FEED_FORWARDS.get(layer.ffn.kind)(layer.ffn.params,
+                                                         joined(layer.prefix, layer.ffn.params.get("prefix", "")), build)
+        self.norms: Dict[str, Any] = {}
+        self.connections: Dict[str, Any] = {}
+        f32 = lambda name: build.loader.get(name).to(torch.float32).contiguous()
+        for which, hc in self._places(layer):
+            norm = layer.norm(which)
+            made = NORMS.get(norm.kind)(norm.params, joined(layer.prefix, p[which]), build)
+            if not getattr(made, "takes_streams", False) or getattr(made, "streams", 1) != self.streams:
+                raise ValueError(f"the hyper block needs norms that read {self.streams} streams, '{norm.kind}' does not")
+            self.norms[which] = made
+            if p.get("learned", True):
+                sub = joined(layer.prefix, p[hc])
+                self.connections[which] = (f32(joined(sub, "in")), f32(joined(sub, "mix")), f32(joined(sub, "out")))
+            else:
+                self.connections[which] = (None, torch.eye(self.streams, dtype=torch.float32, device=build.device),
+                                           torch.ones(self.streams, dtype=torch.float32, device=build.device))
+        self.act_dtype = build.act_dtype
+
+    def cache_spec(self) -> Optional[Any]:
+        return self.mixer.cache_spec()
+
+    def records_cleanly(self) -> bool:
+        return all(says(part, "records_cleanly") for part in (self.mixer, self.ffn, *self.norms.values())
+                   if part is not None)
+
+    def entry_norm(self) -> Any:
+        return self.norms["mixer_norm"]
+
+    def _sublayer(self, stream: ResidualStream, ctx: StepContext, which: str, run) -> None:
+        norm = self.norms[which]
+        w_in, mix, w_out = self.connections[which]
+        hidden = stream.h.shape[1] // self.streams
+        x = ctx.workspace.buffer("block.normed", ctx.num_tokens, hidden, self.act_dtype)
+        norm.apply(stream.h, stream.pending_for(norm), x, stream_weights=w_in)
+        y = run(x)
+        if isinstance(y, tuple):   # (a feed-forward that hands back two updates)
+            first, second = y
+            if second is not None:
+                raise TypeError("the hyper block takes one result a sublayer")
+            y = first
+        stream.stats = None
+        stream.pending = StreamUpdate(y, mix, w_out)
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Any) -> None:
+        self._sublayer(stream, ctx, "mixer_norm", lambda x: self.mixer.forward(x, ctx, cache))
+        if self.ffn is not None:
+            self._sublayer(stream, ctx, "ffn_norm", lambda x: self.ffn.forward(x, ctx))

@@ -38,13 +38,17 @@ class TokenEmbedding(Part):
         self.hidden = int(params["hidden_size"])
         self.table = build.loader.get(params["name"])
         self.scale = float(params.get("scale", 1.0))   # every gathered row is multiplied by it, in float32
+        self.streams = int(params.get("streams", 1))   # a residual of several streams gets the row in every one
         self.bad_id = torch.zeros(1, dtype=torch.int32, device=build.device)
 
     def forward(self, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         """The step function checks ids on the host before it runs.  A caller that comes another way and brings an
         id outside the table gets a row of NaN, which reaches that token's logits (no token is chosen from them),
         never a silent row of zeros; ``saw_bad_id`` tells, at the price of a synchronisation."""
-        kernels.embed_gather(ids, self.table, out, self.bad_id, self.scale)
+        if self.streams > 1:
+            kernels.embed_streams(ids, self.table, out, self.bad_id, self.streams, self.scale)
+        else:
+            kernels.embed_gather(ids, self.table, out, self.bad_id, self.scale)
         return out
 
     def saw_bad_id(self, clear: bool = True) -> bool:

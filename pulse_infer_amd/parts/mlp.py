@@ -39,16 +39,19 @@ class GatedMLP(Part):
     def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
         self.hidden = int(params["hidden_size"])
         self.inter = int(params["intermediate_size"])
-        activation = params.get("activation", "silu")
-        if activation != "silu":
-            raise ValueError(f"gated_mlp has no kernel for activation '{activation}' (only 'silu')")
+        self.activation = params.get("activation", "silu")
+        if self.activation not in kernels.GATE_ACTIVATIONS:
+            raise ValueError(f"gated_mlp has no kernel for activation '{self.activation}' "
+                             f"(known: {sorted(kernels.GATE_ACTIVATIONS)})")
         load = build.loader
         names = {k: joined(prefix, v) for k, v in self.tensor_names(params).items()}
         gate, up = load.get(names["gate"]), load.get(names["up"])
         # gate and up rows alternate in slabs of 16 where the sizes allow it, so that one workgroup of the
         # few-rows product holds a gate slab and its up slab and can apply SwiGLU itself (a layout choice)
+        # (the products that apply the activation on their way out know silu; another activation runs as the plain
+        # product followed by the activation's kernel)
         self.slab = SLAB if (build.mode == "bfloat16" and gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16
-                             and self.inter % SLAB == 0) else 0
+                             and self.inter % SLAB == 0 and self.activation == "silu") else 0
         if self.slab:
             stacked = torch.stack([gate.view(-1, SLAB, self.hidden), up.view(-1, SLAB, self.hidden)], dim=1)
             self.gate_up = Linear(stacked.reshape(2 * self.inter, self.hidden).contiguous(), build.mode)
@@ -85,7 +88,7 @@ class GatedMLP(Part):
         else:
             gu = ws.buffer("mlp.gate_up", tokens, 2 * self.inter, self.act_dtype)
             self.gate_up.forward(x, gu, own=False)   # (the shapes that come here at 17 to 64 rows are those the library wins)
-            kernels.swiglu(gu, z, slab=self.slab)
+            kernels.swiglu(gu, z, slab=self.slab, activation=self.activation)
         out = ws.buffer("mlp.out", tokens, self.hidden, self.act_dtype)
         if residual is not None:
             return self.down.add_into(z, residual, out, ws, next_scale, next_offset, leave_stats)

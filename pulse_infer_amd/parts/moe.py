@@ -10,7 +10,11 @@ token and is added.
 Parameters: ``hidden_size``, ``expert_size``, ``num_experts``, ``num_identity``, ``top``, ``correction`` (whether a
 correction tensor exists), ``shared_size`` (None: no shared expert), ``names``: ``router``, ``correction``,
 ``expert`` (a pattern with ``{e}``), ``gate`` / ``up`` / ``down`` (below an expert's or the shared expert's prefix),
-``shared``.
+``shared``; ``score``: "softmax" (default) or "sigmoid" (s = sigmoid(z), every output by itself); ``renormalize``
+(default True; False: the weights are the chosen scores as they are); ``weight_on``: "output" (default) or "input" (an
+expert is fed weight * x, and the experts' results are added as they are); ``expert_activation``: "silu" (default) or
+"clamped_swish" with ``limit``: g = min(gate x, limit), u = clamp(up x, -limit, limit), down(g * sigmoid(1.702 g) *
+(u + 1)).
 
 The experts' weights are stacked at load time ([experts, rows, columns]).  ``forward`` returns the routed part
 (float32) and the shared expert's part as two updates that the block adds.
@@ -102,6 +106,23 @@ class RoutedExperts(Part):
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
         shared = self._shared_params(params)
         self.shared = GatedMLP(shared, joined(prefix, n["shared"]), build) if shared is not None else None
+        self.score = params.get("score", "softmax")
+        if self.score not in kernels.ROUTER_SCORES:
+            raise ValueError(f"a router scores by {sorted(kernels.ROUTER_SCORES)}, not '{self.score}'")
+        self.renormalize = bool(params.get("renormalize", True))
+        weight_on = params.get("weight_on", "output")
+        if weight_on not in ("output", "input"):
+            raise ValueError(f"an expert's weight goes on its 'output' or its 'input', not '{weight_on}'")
+        self.weight_on_input = weight_on == "input"
+        if self.weight_on_input and self.identity:
+            raise ValueError("identity experts take their weight on the output")
+        self.expert_activation = params.get("expert_activation", "silu")
+        if self.expert_activation not in kernels.EXPERT_ACTIVATIONS:
+            raise ValueError(f"experts know the activations {sorted(kernels.EXPERT_ACTIVATIONS)}, not "
+                             f"'{self.expert_activation}'")
+        self.limit = float(params.get("limit", 0.0))
+        if self.expert_activation == "clamped_swish" and not self.limit > 0.0:
+            raise ValueError("the clamped activation needs a positive limit")
         self.act_dtype = build.act_dtype
         self.device = build.device
 
@@ -113,7 +134,8 @@ class RoutedExperts(Part):
         ws = ctx.workspace
         idx = ws.buffer("moe.idx", tokens, self.top, torch.int32)
         weight = ws.buffer("moe.weight", tokens, self.top, torch.float32)
-        kernels.moe_router(x, self.router, self.correction, self.top, idx, weight)   # logits in float32 inside
+        kernels.moe_router(x, self.router, self.correction, self.top, idx, weight, score=self.score,
+                           renormalize=self.renormalize)   # logits in float32 inside
         act = ws.buffer("moe.act", tokens * self.top, self.ff, self.act_dtype)
         routed = ws.buffer("moe.out", tokens, self.hidden, torch.float32)
         if kernels.moe_grouped_takes(x, self.w_gate, self.w_down):
@@ -123,9 +145,12 @@ class RoutedExperts(Part):
             rows = kernels.MOE_TILE_ROWS[1] if pairs >= 64 * self.experts else kernels.MOE_TILE_ROWS[0]
             y = ws.buffer("moe.y", pairs, self.hidden, torch.float32)
             ints = ws.buffer("moe.ints", 2 * pairs + 3 * kernels.moe_max_tiles(pairs, self.experts, rows) + 1, 1, torch.int32)
-            kernels.moe_grouped(x, self.w_gate, self.w_up, self.w_down, idx, weight, act, y, routed, ints.view(-1), rows)
+            kernels.moe_grouped(x, self.w_gate, self.w_up, self.w_down, idx, weight, act, y, routed, ints.view(-1), rows,
+                                weight_on_input=self.weight_on_input, activation=self.expert_activation,
+                                limit=self.limit)
         else:
-            kernels.moe_gate_up(x, self.w_gate, self.w_up, idx, act)
-            kernels.moe_down(x, act, self.w_down, idx, weight, routed)
+            kernels.moe_gate_up(x, self.w_gate, self.w_up, idx, act, in_weight=weight if self.weight_on_input else None,
+                                activation=self.expert_activation, limit=self.limit)
+            kernels.moe_down(x, act, self.w_down, idx, None if self.weight_on_input else weight, routed)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
         return routed, shared

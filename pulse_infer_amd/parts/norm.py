@@ -12,7 +12,7 @@ import torch
 
 from ..ops import kernels
 from ..weights.store import TensorSpec
-from .base import NORMS, BuildContext, LazyNorm, Part, RowStats, joined
+from .base import NORMS, BuildContext, LazyNorm, Part, RowStats, StreamUpdate, joined
 
 
 @NORMS.register("rmsnorm")
@@ -49,3 +49,50 @@ class RMSNorm(Part):
         if stats.rounded is None or stats.scaled_by is not self.weight or stats.offset != self.weight_offset:
             return None
         return LazyNorm(stats.rounded, stats.sumsq, self.eps, h, self)
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Part):
+    """y = (x - mean) / sqrt(var + eps) * w + b, var the mean of the squared deviations; float32 inside, one rounding.
+
+    Parameters: ``size``, ``eps``; ``tensor`` / ``bias_tensor``: the tensors' names below the norm's prefix (defaults
+    "weight" and "bias"; "": the prefix itself is the tensor's name); ``bias`` False: no bias; ``streams`` (default
+    1): the residual it reads holds that many rows a token side by side, and the norm reads their weighted sum
+    (``stream_weights`` of ``apply``; None: the plain sum)."""
+
+    records_cleanly = True
+    takes_streams = True    # ``apply`` takes a ``StreamUpdate`` as the update and does it on the way
+
+    @classmethod
+    def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
+        out = {params.get("tensor", "weight"): TensorSpec((params["size"],), kind="norm")}
+        if params.get("bias", True):
+            out[params.get("bias_tensor", "bias")] = TensorSpec((params["size"],), kind="linear", fan_in=100)
+        return out
+
+    def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
+        self.size = int(params["size"])
+        self.eps = float(params["eps"])
+        self.streams = int(params.get("streams", 1))
+        self.weight = build.loader.get(joined(prefix, params.get("tensor", "weight")))
+        self.bias = None
+        if params.get("bias", True):
+            self.bias = build.loader.get(joined(prefix, params.get("bias_tensor", "bias")))
+            if self.bias.dtype != self.weight.dtype:
+                self.bias = self.bias.to(self.weight.dtype)
+
+    def apply(self, h: torch.Tensor, delta: Any, out: torch.Tensor, rows: Optional[torch.Tensor] = None,
+              stream_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """out = norm(sum_s weights[s] * h_s) after ``delta`` has gone into h: a ``StreamUpdate`` (done by the same
+        kernel), a tensor of h's shape (added first), or None."""
+        update = None
+        if isinstance(delta, StreamUpdate):
+            if rows is None:
+                update = (delta.y, delta.mix, delta.out)
+            else:
+                delta.apply_to(h)
+        elif delta is not None:
+            kernels.residual_add(h, delta)
+        kernels.streams_step(h, self.streams, update=update, in_weight=stream_weights,
+                             norm=("layernorm", self.weight, self.bias, self.eps), out=out, rows=rows)
+        return out

@@ -59,7 +59,7 @@ def check(name, args):
             need(int(ent.tensor[:tokens].max()) < bt.tensor.shape[0] and bt.tensor.shape[1] == width, "table")
             need(int(pos.tensor[:tokens].max()) // page < width, "a position beyond the table")
     elif name == "pulse_attn_generic":
-        (q, qs, out, os_, _, _, _, _, pos, ent, bt, width, tokens, nq, _, d, page, _, _, _, gate, gs, _) = args
+        (q, qs, out, os_, _, _, _, _, pos, ent, bt, width, tokens, nq, _, d, page, _, _, _, gate, gs, _, _, _, _) = args
         tokens, nq, d = val(tokens), val(nq), val(d)
         need(room(q) >= (tokens - 1) * val(qs) + nq * d and room(out) >= (tokens - 1) * val(os_) + nq * d, "q / out")
         need(gate.tensor is None or room(gate) >= (tokens - 1) * val(gs) + nq, "gate")
@@ -122,7 +122,7 @@ def check(name, args):
         else:
             need(room(c) >= (m - 1) * val(ldc) + n, "out")
     elif name == "pulse_swiglu":
-        gu, out, _, tokens, inter, _, _ = args
+        gu, out, _, tokens, inter, _, _, _ = args
         need(room(gu) >= val(tokens) * 2 * val(inter) and room(out) >= val(tokens) * val(inter), "operands")
     elif name == "pulse_embed_gather":
         ids, _, _, out, tokens, hidden, _, _, _, _ = args
