@@ -55,13 +55,14 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
     p.add_argument("--model", choices=sorted(SHAPES), default="8b", help="layer sizes: Qwen3-8B (the default), 14B or 32B")
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has, if memory or time needs it")
-    p.add_argument("--workload", choices=["decode", "serving", "long-prompt", "dirozen", "kesovik"], default="decode",
+    p.add_argument("--workload", choices=["decode", "serving", "long-prompt", "dirozen", "kesovik", "tipidra"], default="decode",
                    help="decode: fixed batch at a fixed context; serving: continuous batching of requests with "
                         "seeded prompt lengths, chunked prefill mixed with decoding; long-prompt: one prompt of "
                         "--prompt-tokens tokens in portions of --chunk tokens; dirozen / kesovik: decoding and prefill of "
-                        "that design beside Qwen3 layers of equal sizes, with both models' time by entry point")
-    p.add_argument("--compare-layers", type=int, default=4, help="dirozen, kesovik: layers of the two models that are compared")
-    p.add_argument("--compare-sizes", default="2k,4k,5k", help="dirozen, kesovik: which of the layer sizes 2k, 4k, 5k (widths) to run")
+                        "that design beside Qwen3 layers of equal sizes, with both models' time by entry point; "
+                        "tipidra: the same beside Kesovik and Qwen3 layers")
+    p.add_argument("--compare-layers", type=int, default=4, help="dirozen, kesovik, tipidra: layers of the models that are compared")
+    p.add_argument("--compare-sizes", default="2k,4k,5k", help="dirozen, kesovik, tipidra: which of the layer sizes 2k, 4k, 5k (widths) to run")
     p.add_argument("--prompt-tokens", type=int, default=16384, help="long-prompt: length of the prompt")
     p.add_argument("--requests", type=int, default=32, help="serving: number of requests")
     p.add_argument("--prompt-range", type=int, nargs=2, default=[128, 2048], help="serving: prompt lengths drawn from [lo, hi]")
@@ -252,6 +253,22 @@ def kesovik_layers(size, layers):
     return [turn[i % len(turn)] for i in range(layers)]
 
 
+def tipidra_layers(size, layers):
+    """Tipidra layers at the comparison's sizes, in turn: attention (heads as Qwen3's, a score cap, sinks, a gate a
+    channel, a rotation on half of a head) with a dense feed-forward; a selective state-space mixer (twice the width
+    inside, 16 states a channel, step sizes of rank width / 16, 4 taps) with routed experts; attention with routed
+    experts; the state-space mixer with a dense feed-forward.  The routed feed-forward has 16 experts an eighth as
+    wide as the dense one, 4 chosen a token: half of the dense feed-forward's arithmetic a token."""
+    attention = {"dim": size["dim"], "heads": size["heads"], "kv_heads": size["kv_heads"], "vdim": size["dim"],
+                 "rot": {"base": 1e6, "dims": size["dim"] // 2}, "scale": size["dim"] ** -0.5, "softcap": 50.0}
+    ssm = {"inner": 2 * size["width"], "state": 16, "dt_rank": size["width"] // 16, "conv": 4}
+    dense = {"ff": size["ff"], "kind": "dense"}
+    routed = {"expert": {"ff": size["ff"] // 8, "limit": 7.0}, "kind": "moe", "router": {"experts": 16, "top": 4}}
+    turn = [{"type": "attention", "mixer": attention, "mlp": dense}, {"type": "mamba1", "mixer": ssm, "mlp": routed},
+            {"type": "attention", "mixer": attention, "mlp": routed}, {"type": "mamba1", "mixer": ssm, "mlp": dense}]
+    return [turn[i % len(turn)] for i in range(layers)]
+
+
 def dirozen_compare(args, design: str = "dirozen") -> int:
     """Dirozen (or, with ``design`` "kesovik", Kesovik) beside Qwen3 layers of equal sizes (random weights, ``--compare-layers`` layers, a vocabulary of
     32,000): decoding at batch 1 / 8 / 32 with contexts ending at ``--context`` and a prompt of ``--prefill-tokens``
@@ -260,7 +277,7 @@ def dirozen_compare(args, design: str = "dirozen") -> int:
     line."""
     import torch
 
-    from pulse_infer_amd.config import DirozenConfig, KesovikConfig, Qwen3Config
+    from pulse_infer_amd.config import DirozenConfig, KesovikConfig, Qwen3Config, TipidraConfig
     from pulse_infer_amd.engine.engine import ContinuousBatchEngine
     from pulse_infer_amd.engine.runner import StepEntry
     from pulse_infer_amd.models.causal_lm import expected_tensors
@@ -290,11 +307,17 @@ def dirozen_compare(args, design: str = "dirozen") -> int:
                  "mlp": {"ff": size["ff"], "kind": "dense"}}
         dirozen = DirozenConfig.from_dict({"architecture": "Dirozen", "vocab": vocab, "width": size["width"],
                                            "norm": {"eps": 1e-6}, "layers": [entry] * layers}, "<bench>")
-        if design == "kesovik":
+        if design in ("kesovik", "tipidra"):
             kesovik = KesovikConfig.from_dict({
                 "architecture": "Kesovik", "vocab": vocab, "width": size["width"], "norm": {"eps": 1e-6},
                 "embedding": {"scale": 1.0}, "postln_alpha": 2.0, "logit_softcap": 30.0,
                 "layers": kesovik_layers(size, layers)}, "<bench>")
+            if design == "tipidra":
+                tipidra = TipidraConfig.from_dict({
+                    "architecture": "Tipidra", "vocab": vocab, "width": size["width"], "norm": {"eps": 1e-6},
+                    "embedding": {"scale": 1.0}, "logit_softcap": 30.0, "streams": 4,
+                    "layers": tipidra_layers(size, layers)}, "<bench>")
+                return {"tipidra": tipidra, "kesovik": kesovik, "qwen3": qwen}
             return {"kesovik": kesovik, "qwen3": qwen}
         return {"dirozen": dirozen, "qwen3": qwen}
 
@@ -379,23 +402,27 @@ def dirozen_compare(args, design: str = "dirozen") -> int:
         torch.cuda.empty_cache()
         return out
 
-    record = {"metric": f"{design}_beside_qwen3_layers", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype,
+    record = {"metric": f"{design}_beside_{'kesovik_and_' if design == 'tipidra' else ''}qwen3_layers", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype,
               "data": "synthetic", "layers": layers, "vocab": vocab, "context": args.context, "sizes": {}}
     for name, size in DIROZEN_SIZES.items():
         if name not in args.compare_sizes.split(","):
             continue
         both = {model: measure(cfg) for model, cfg in configs(size).items()}
-        ratio = {k: round(both[design][k]["tokens_per_s"] / both["qwen3"][k]["tokens_per_s"], 3)
-                 for k in both[design] if "tokens_per_s" in both[design][k]}
-        record["sizes"][name] = dict(size, **both, **{f"{design}_over_qwen3": ratio})
+        ratios = {}
+        for other in both:
+            if other != design:
+                ratios[f"{design}_over_{other}"] = {
+                    k: round(both[design][k]["tokens_per_s"] / both[other][k]["tokens_per_s"], 3)
+                    for k in both[design] if "tokens_per_s" in both[design][k]}
+        record["sizes"][name] = dict(size, **both, **ratios)
     print(json.dumps(record))
     return 0
 
 
 def main() -> int:
     args = parse_args()
-    if args.workload == "kesovik":
-        return dirozen_compare(args, "kesovik")
+    if args.workload in ("kesovik", "tipidra"):
+        return dirozen_compare(args, args.workload)
     if args.workload == "dirozen":
         if args.gpus != 1:
             print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")

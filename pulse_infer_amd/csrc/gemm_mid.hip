@@ -52,6 +52,14 @@ __device__ __forceinline__ bf16x8 zeros8() {
 
 // NW wavefronts of 16 weight rows each a workgroup; MT tiles of 16 rows of X; KC k a chunk (steps of 32); RING
 // register sets of weight chunks (a wavefront has RING - 1 chunks of its 16 weight rows in flight).
+// The gate's activation of the epilogues that multiply gate and up: silu, or with bit ACT_GELU of `mode` set (the
+// output modes proper stay below it) the tanh form of gelu.
+constexpr int ACT_GELU = 8;
+__device__ __forceinline__ float gate_activation(float g, int mode) {
+    if (mode & ACT_GELU) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.0f + expf(-g));
+}
+
 template <int NW, int MT, int KC, bool SWIGLU, int RING>
 __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* __restrict__ X, int64_t ldx,
                                                                     const bf16_t* __restrict__ W, int64_t ldw,
@@ -230,7 +238,7 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const float g = acc[mt][i];
-                    v[i] = (__bf16)(g / (1.0f + expf(-g)) * up[i]);
+                    v[i] = (__bf16)(gate_activation(g, mode) * up[i]);
                 }
                 *reinterpret_cast<bf16x4*>(dst) = v;   // N is a multiple of 32: whole groups of four
             }
@@ -306,6 +314,8 @@ extern "C" int pulse_gemm_mid(const void* X, int64_t ldx, const void* W, int64_t
     } else {
         PULSE_REQUIRE(ldc >= N, "gemm_mid: output row stride too small");
     }
+    PULSE_REQUIRE(swiglu >= 0 && swiglu <= 2, "gemm_mid: swiglu is 0 (none), 1 (silu) or 2 (gelu, tanh form), got %d", swiglu);
+    if (swiglu == 2) mode |= ACT_GELU;
     const bf16_t* x = static_cast<const bf16_t*>(X);
     const bf16_t* w = static_cast<const bf16_t*>(W);
     const int k_len = K / splits;

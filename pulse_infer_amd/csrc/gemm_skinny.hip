@@ -67,6 +67,14 @@ __device__ __forceinline__ int row_shift_left(int v, int n) {
 // takes the new values once more, each multiplied by its column's `copy_scale` (that norm's weight; null: 1) and
 // rounded to bfloat16 (that product's input).  `row_scale` (one factor for each of at most 16 rows) multiplies the
 // sums before anything else is done with them.
+// The gate's activation of the epilogues that multiply gate and up: silu, or with bit ACT_GELU of `mode` set (the
+// output modes proper stay below it) the tanh form of gelu.
+constexpr int ACT_GELU = 8;
+__device__ __forceinline__ float gate_activation(float g, int mode) {
+    if (mode & ACT_GELU) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.0f + expf(-g));
+}
+
 template <int SLABS, int MT, int KW, bool SWIGLU>
 __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void* __restrict__ C, int64_t ldc, int M, int N,
                                          int n_base, int mode, int tid, float* __restrict__ sumsq = nullptr, int parts = 0,
@@ -131,7 +139,7 @@ __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void*
             const int m = mt * 16 + m_in;
             const int n = n_base / 2 + pair * 16 + n_in;
             if (m < M && 2 * n < N) {  // N counts gate and up rows together
-                const float v = g / (1.0f + expf(-g)) * u;
+                const float v = gate_activation(g, mode) * u;
                 static_cast<bf16_t*>(C)[static_cast<int64_t>(m) * ldc + n] = f32_to_bf16(v);
             }
         }
@@ -530,6 +538,8 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
         PULSE_REQUIRE(ldc >= N, "gemm_skinny: output row stride too small");
     }
     if (M == 0) return 0;
+    PULSE_REQUIRE(swiglu >= 0 && swiglu <= 2, "gemm_skinny: swiglu is 0 (none), 1 (silu) or 2 (gelu, tanh form), got %d", swiglu);
+    if (swiglu == 2) mode |= ACT_GELU;
     const bf16_t* x = static_cast<const bf16_t*>(X);
     RowScale scale{scale_sumsq, scale_parts, scale_eps};
     const int parts_out = (N + 15) / 16;

@@ -128,6 +128,18 @@ def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
 GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
 
 
+def gate_code(swiglu) -> int:
+    """What the products that multiply gate and up on their way out are told: 0 none, 1 silu (True), 2 the tanh form
+    of gelu."""
+    if not swiglu:
+        return 0
+    if swiglu is True or swiglu == "silu":
+        return 1
+    if swiglu == "gelu_tanh":
+        return 2
+    raise KernelError(f"a gated product knows the activations {sorted(GATE_ACTIVATIONS)}, not {swiglu!r}")
+
+
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor, slab: int = 0, activation: str = "silu") -> None:
     """out[t, i] = act(gate) * up, act silu or the tanh form of gelu; gate_up holds [gate | up] halves (slab 0) or
     alternating slabs of ``slab`` columns."""
@@ -254,7 +266,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool =
               "gemm_skinny: the row sums of squares must be a contiguous, 16-byte aligned float32 [M, parts]")
         scale_parts = scale_sumsq.shape[1]
     call("pulse_gemm_skinny_fused", _ptr(a), _i64(ldx), _ptr(w), _i64(w.stride(0) if n > 1 else k), _ptr(out),
-         _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0),
+         _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(gate_code(swiglu)),
          _i32(tune), _ptr(scale_sumsq), _i32(scale_parts), _f32(scale_eps), _ptr(sumsq_out), _ptr(copy_out),
          _i64(ldcopy), _ptr(copy_scale), _f32(copy_offset), _stream(), label=f"N={n} K={k}")
 
@@ -395,7 +407,7 @@ def gemm_mid(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool =
               and out.shape[1] == cols and out.stride(1) == 1, f"gemm_mid: out must be bfloat16 [{m}, {cols}]")
         mode, ldc = 0, (out.stride(0) if m > 1 else cols)
     call("pulse_gemm_mid", _ptr(a), _i64(a.stride(0) if m > 1 else k), _ptr(w), _i64(w.stride(0) if n > 1 else k),
-         _ptr(out), _i64(ldc), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0), _i32(splits), _i32(waves),
+         _ptr(out), _i64(ldc), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(gate_code(swiglu)), _i32(splits), _i32(waves),
          _stream(), label=f"N={n} K={k}")
 
 

@@ -16,7 +16,7 @@ Three products stand behind it:
 from __future__ import annotations
 
 import os
-from typing import Optional
+from typing import Any, Optional
 
 import torch
 
@@ -55,7 +55,7 @@ class Linear:
         return (self.library and kernels.gemm_skinny_fusable(x.shape[0], n, self.in_features)
                 and x.x.dtype == torch.bfloat16 and kernels.gemm_skinny_ok(x.x, self.weight))
 
-    def forward(self, x, out: torch.Tensor, rows: Optional[int] = None, swiglu: bool = False,
+    def forward(self, x, out: torch.Tensor, rows: Optional[int] = None, swiglu: Any = False,
                 own: bool = True) -> torch.Tensor:
         """``out`` [M, out_features] receives the product; its storage type is bfloat16 or float32.  ``x`` may be a
         ``LazyNorm`` that ``takes_lazy`` accepted.  ``swiglu``: few rows of a slab-interleaved gate/up weight only.
@@ -65,13 +65,15 @@ class Linear:
         if isinstance(x, LazyNorm):
             kernels.gemm_skinny(x.x, w, out, swiglu=swiglu, row_scale=(x.sumsq, x.eps))
             return out
-        if swiglu:
+        if swiglu:   # (True, or the gate's activation by name where it is not silu; the tiled product knows silu)
             if x.shape[0] > self.MID_ROWS[1]:
+                if kernels.gate_code(swiglu) != 1:
+                    raise ValueError("the tiled product applies silu only")
                 kernels.gemm_tile(x, w, out, swiglu=True)
             elif x.shape[0] > kernels.SKINNY_FAST_ROWS:
-                kernels.gemm_mid(x, w, out, swiglu=True, waves=self.swiglu_waves_for(x.shape[0]) or 4)
+                kernels.gemm_mid(x, w, out, swiglu=swiglu, waves=self.swiglu_waves_for(x.shape[0]) or 4)
             else:
-                kernels.gemm_skinny(x, w, out, swiglu=True)
+                kernels.gemm_skinny(x, w, out, swiglu=swiglu)
             return out
         if self.library and x.dtype == torch.bfloat16:
             few = x.shape[0] <= kernels.SKINNY_FAST_ROWS

@@ -48,10 +48,8 @@ class GatedMLP(Part):
         gate, up = load.get(names["gate"]), load.get(names["up"])
         # gate and up rows alternate in slabs of 16 where the sizes allow it, so that one workgroup of the
         # few-rows product holds a gate slab and its up slab and can apply SwiGLU itself (a layout choice)
-        # (the products that apply the activation on their way out know silu; another activation runs as the plain
-        # product followed by the activation's kernel)
         self.slab = SLAB if (build.mode == "bfloat16" and gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16
-                             and self.inter % SLAB == 0 and self.activation == "silu") else 0
+                             and self.inter % SLAB == 0) else 0
         if self.slab:
             stacked = torch.stack([gate.view(-1, SLAB, self.hidden), up.view(-1, SLAB, self.hidden)], dim=1)
             self.gate_up = Linear(stacked.reshape(2 * self.inter, self.hidden).contiguous(), build.mode)
@@ -76,14 +74,16 @@ class GatedMLP(Part):
         z = ws.buffer("mlp.act", tokens, self.inter, self.act_dtype)
         if isinstance(x, LazyNorm) and not (self.slab and self.gate_up.takes_lazy(x)):
             x = x.materialize(ws.buffer("mlp.normed", tokens, self.hidden, self.act_dtype))
+        gated = True if self.activation == "silu" else self.activation   # what the fused epilogues are told
         if isinstance(x, LazyNorm):
-            self.gate_up.forward(x, z, swiglu=True)
-        elif (self.slab and tokens <= kernels.SKINNY_FAST_ROWS and kernels.gemm_skinny_ok(x, self.gate_up.weight)):
-            self.gate_up.forward(x, z, swiglu=True)
+            self.gate_up.forward(x, z, swiglu=gated)
+        elif (self.slab and tokens <= kernels.SKINNY_FAST_ROWS and kernels.gemm_skinny_ok(x, self.gate_up.weight)
+              and (2 * self.inter) % 32 == 0):
+            self.gate_up.forward(x, z, swiglu=gated)
         elif (self.slab and self.gate_up.takes_mid(x) and (2 * self.inter) % 32 == 0
               and kernels.gemm_mid_takes(tokens, 2 * self.inter, self.hidden)):
-            self.gate_up.forward(x, z, swiglu=True)   # 17 to 64 rows: X shared through LDS, SwiGLU in the epilogue
-        elif self.slab and self.gate_up.takes_tiles(x, swiglu=True):
+            self.gate_up.forward(x, z, swiglu=gated)   # 17 to 64 rows: X shared through LDS, SwiGLU in the epilogue
+        elif self.slab and self.activation == "silu" and self.gate_up.takes_tiles(x, swiglu=True):
             self.gate_up.forward(x, z, swiglu=True)   # many rows: output tiles on the matrix cores, SwiGLU on the way out
         else:
             gu = ws.buffer("mlp.gate_up", tokens, 2 * self.inter, self.act_dtype)
