@@ -13,9 +13,10 @@
 //     dt      = softplus(dt_raw[t, c] + dt_bias[c])
 //     S[c, n] = exp(dt * A[c, n]) * S[c, n] + dt * x[t, c] * B[t, n],     A = -exp(A_log)
 //     y[t, c] = (sum_n S[c, n] * C[t, n] + D[c] * x[t, c]) * silu(z[t, c])
-// L lanes share a channel's N states (n = lane + L * j) and add their shares of y through lane exchanges; the same
-// kernel serves prompt portions, decoded tokens and mixed batches, so a prompt cut anywhere goes through the same
-// arithmetic.  State, step sizes, decays, exponentials and sums are float32 whatever the storage type of the rows.
+// L lanes share a channel's N states (n = lane + L * j) and add their shares of y through lane exchanges; the
+// tokens' values are staged through LDS a chunk at a time while the next chunk is fetched; the same kernel serves
+// prompt portions, decoded tokens and mixed batches, so a prompt cut anywhere goes through the same arithmetic.
+// State, step sizes, decays, exponentials and sums are float32 whatever the storage type of the rows.
 #include "common.h"
 
 #include <math.h>
@@ -25,8 +26,19 @@ namespace {
 constexpr int MAX_TAPS = 16;
 constexpr int MAX_NS = 16;   // states a lane
 
-__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
-__device__ __forceinline__ float softplus_f(float v) { return v > 20.f ? v : log1pf(expf(v)); }
+// silu and softplus in float32: with the library's accurate functions where the rows are float32, with the
+// hardware's exponential, logarithm and reciprocal (a few units in the last place, a handful of instructions) where
+// the result is rounded to bfloat16 or feeds bfloat16 rows anyway.
+template <typename TX>
+__device__ __forceinline__ float silu_f(float v) {
+    if constexpr (sizeof(TX) == 4) return v / (1.0f + expf(-v));
+    else return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+}
+template <typename TX>
+__device__ __forceinline__ float softplus_f(float v) {
+    if constexpr (sizeof(TX) == 4) return v > 20.f ? v : log1pf(expf(v));
+    else return v > 20.f ? v : __logf(1.0f + __expf(v));
+}
 
 struct ConvArgs {
     int channels, taps, n_state, state_row;   // state_row = n_state + taps - 1
@@ -59,7 +71,56 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const TX* __restrict__
         else if (q >= 0) v = tail[(K - 1) - (start - q)];   // start > 0 here
         acc = fmaf(to_f32<TW>(taps[static_cast<int64_t>(c) * K + j]), v, acc);
     }
-    out[static_cast<int64_t>(t) * a.out_stride + c] = from_f32<TX>(silu_f(acc));
+    out[static_cast<int64_t>(t) * a.out_stride + c] = from_f32<TX>(silu_f<TX>(acc));
+}
+
+// The same for bfloat16 rows whose sizes allow 16-byte accesses: a thread takes 8 neighbouring channels of a token.
+template <typename TW>
+__global__ __launch_bounds__(256) void causal_conv_bf16x8_kernel(const bf16_t* __restrict__ in, const TW* __restrict__ taps,
+                                                                 const TW* __restrict__ bias, bf16_t* __restrict__ out,
+                                                                 const float* __restrict__ state,
+                                                                 const int* __restrict__ positions,
+                                                                 const int* __restrict__ token_entry,
+                                                                 const int* __restrict__ entry_start,
+                                                                 const int* __restrict__ entry_first_row,
+                                                                 const int* __restrict__ entry_slot, ConvArgs a) {
+    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    const int t = blockIdx.y;
+    if (c >= a.channels) return;
+    const int e = token_entry[t];
+    const int start = entry_start[e], row0 = entry_first_row[e];
+    const int pos = positions[t];
+    const int K = a.taps;
+    const float* tail = state + (static_cast<int64_t>(entry_slot[e]) * a.channels + c) * a.state_row + a.n_state;
+    float acc[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc[u] = bias ? to_f32<TW>(bias[c + u]) : 0.f;
+    for (int j = 0; j < K; ++j) {
+        const int q = pos - (K - 1) + j;
+        float v[8];
+        if (q >= start) {
+            const pulse_i32x4 raw = *reinterpret_cast<const pulse_i32x4*>(in + static_cast<int64_t>(row0 + q - start) * a.in_stride + c);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t two = static_cast<uint32_t>(raw[u]);
+                v[2 * u] = __uint_as_float(two << 16);
+                v[2 * u + 1] = __uint_as_float(two & 0xffff0000u);
+            }
+        } else if (q >= 0) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = tail[static_cast<int64_t>(u) * a.state_row + (K - 1) - (start - q)];
+        } else {
+            continue;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc[u] = fmaf(to_f32<TW>(taps[static_cast<int64_t>(c + u) * K + j]), v[u], acc[u]);
+    }
+    uint32_t packed[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        packed[u] = static_cast<uint32_t>(f32_to_bf16(silu_f<bf16_t>(acc[2 * u]))) |
+                    (static_cast<uint32_t>(f32_to_bf16(silu_f<bf16_t>(acc[2 * u + 1]))) << 16);
+    *reinterpret_cast<uint4*>(out + static_cast<int64_t>(t) * a.out_stride + c) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
 }
 
 template <typename TX>
@@ -87,83 +148,157 @@ __global__ __launch_bounds__(256) void conv_tail_kernel(const TX* __restrict__ i
 }
 
 struct ScanArgs {
-    int channels, n_state, state_row, lanes, entries;
+    int channels, n_state, state_row, entries;
     int64_t x_stride, dt_stride, bc_stride, z_stride, y_stride;
     int b0, c0;   // columns of B and C in a row of bc
 };
 
-template <typename TX, typename TW, int NS>
-__global__ __launch_bounds__(256) void selective_scan_kernel(const TX* __restrict__ x, const TX* __restrict__ dt_raw,
-                                                             const TW* __restrict__ dt_bias,
-                                                             const TW* __restrict__ a_log, const TX* __restrict__ bc,
-                                                             const TW* __restrict__ d_skip, const TX* __restrict__ z,
-                                                             TX* __restrict__ y, float* __restrict__ state,
-                                                             const int* __restrict__ entry_start,
-                                                             const int* __restrict__ entry_first_row,
-                                                             const int* __restrict__ entry_slot, ScanArgs a) {
-    const int L = a.lanes;
-    const int per_block = blockDim.x / L;
-    const int sub = threadIdx.x % L;
-    const int c = blockIdx.x * per_block + threadIdx.x / L;
+constexpr int SCAN_THREADS = 256;
+
+// A value of every lane of a group of L neighbouring lanes (L a power of two up to 16) summed over the group, left
+// in all of them: exchanges inside a quad, then mirrored halves of a row of 16 lanes (no LDS traffic).
+template <int CTRL>
+__device__ __forceinline__ float lane_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+template <int L>
+__device__ __forceinline__ float group_sum(float v) {
+    if constexpr (L >= 2) v += lane_move<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+    if constexpr (L >= 4) v += lane_move<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+    if constexpr (L >= 8) v += lane_move<0x141>(v);   // row_half_mirror: the other quad of a half row
+    if constexpr (L >= 16) v += lane_move<0x140>(v);  // row_mirror: the other half of a row
+    return v;
+}
+
+// exp of the recurrence: the accurate one where the rows are float32, the fast one (one instruction behind a
+// multiplication, a few units in the last place) where they are bfloat16 anyway.
+template <typename TX>
+__device__ __forceinline__ float decay_exp(float v) {
+    if constexpr (sizeof(TX) == 4) return expf(v);
+    else return __expf(v);
+}
+
+// A workgroup owns CH = 256 / L neighbouring channels of one entry; the L lanes of a channel hold NS neighbouring
+// states each (n = lane * NS + j; NP = L * NS >= N).  Few lanes a channel keep the work that a token costs a
+// channel once (its values read, the lanes' sums brought together, the result stored) small beside the updates.
+// The tokens come through LDS a chunk of CHUNK at a time, a row of W = 3 CH + 2 NP floats a token:
+//   [x: CH | dt = softplus(dt_raw + bias): CH | silu(z): CH | B: NP | C: NP]
+// so that step sizes and gates are computed once a (token, channel) and B and C are read from memory once a
+// workgroup.  While a chunk is walked the next one is on its way into registers, as loaded (nothing is computed
+// with a value before the chunk in hand is through); the chunk's outputs leave together.
+template <typename TX, typename TW, int NS, int L>
+__global__ __launch_bounds__(SCAN_THREADS) void selective_scan_kernel(
+        const TX* __restrict__ x, const TX* __restrict__ dt_raw, const TW* __restrict__ dt_bias,
+        const TW* __restrict__ a_log, const TX* __restrict__ bc, const TW* __restrict__ d_skip,
+        const TX* __restrict__ z, TX* __restrict__ y, float* __restrict__ state, const int* __restrict__ entry_start,
+        const int* __restrict__ entry_first_row, const int* __restrict__ entry_slot, ScanArgs a) {
+    constexpr int CH = SCAN_THREADS / L;
+    constexpr int NP = L * NS;
+    constexpr int W = 3 * CH + 2 * NP;
+    constexpr int CHUNK = L == 16 ? 16 : 1024 / CH;
+    constexpr int XS = CHUNK * CH / SCAN_THREADS;                          // values of x (dt, z) a thread stages
+    constexpr int BS = (CHUNK * 2 * NP + SCAN_THREADS - 1) / SCAN_THREADS;   // values of B and C
+    __shared__ __attribute__((aligned(16))) float rows_s[CHUNK * W];
+    __shared__ float y_s[CHUNK * CH];
+    __shared__ float bias_s[CH];
+    const int tid = threadIdx.x;
+    const int sub = tid % L, ch = tid / L;
+    const int c0 = blockIdx.x * CH;
+    const int c = c0 + ch;
     const int e = blockIdx.y;
     const bool live = c < a.channels;
     const int cc = live ? c : a.channels - 1;   // idle lanes walk along (the lane exchanges want whole wavefronts)
     const int start = entry_start[e], row0 = entry_first_row[e];
     const int count = entry_first_row[e + 1] - row0;
     const int N = a.n_state;
+    if (tid < CH) bias_s[tid] = (dt_bias && c0 + tid < a.channels) ? to_f32<TW>(dt_bias[c0 + tid]) : 0.f;
     float* srow = state + (static_cast<int64_t>(entry_slot[e]) * a.channels + cc) * a.state_row;
     float S[NS], A[NS];
 #pragma unroll
     for (int j = 0; j < NS; ++j) {
-        const int n = sub + L * j;
+        const int n = sub * NS + j;
         A[j] = n < N ? -expf(to_f32<TW>(a_log[static_cast<int64_t>(cc) * N + n])) : 0.f;
         S[j] = (n < N && start > 0) ? srow[n] : 0.f;
     }
-    const float bias = dt_bias ? to_f32<TW>(dt_bias[cc]) : 0.f;
     const float dsk = d_skip ? to_f32<TW>(d_skip[cc]) : 0.f;
-    // the next token's values are asked for while this token's are worked on
-    float xv, dv, zv, Bn[NS], Cn[NS];
-    auto fetch = [&](int i, float& fx, float& fd, float& fz, float* fb, float* fc) {
-        const int64_t row = row0 + i;
-        fx = to_f32<TX>(x[row * a.x_stride + cc]);
-        fd = to_f32<TX>(dt_raw[row * a.dt_stride + cc]);
-        fz = z ? to_f32<TX>(z[row * a.z_stride + cc]) : 0.f;
-        const TX* r = bc + row * a.bc_stride;
+
+    TX sx[XS], sd[XS], sz[XS], sb[BS];
+    const TX zero = from_f32<TX>(0.f);
+    auto fetch = [&](int base, int tokens) {
 #pragma unroll
-        for (int j = 0; j < NS; ++j) {
-            const int n = sub + L * j;
-            fb[j] = n < N ? to_f32<TX>(r[a.b0 + n]) : 0.f;
-            fc[j] = n < N ? to_f32<TX>(r[a.c0 + n]) : 0.f;
+        for (int j = 0; j < XS; ++j) {
+            const int i = tid + SCAN_THREADS * j;
+            const int tt = i / CH, k = c0 + i % CH;
+            const bool ok = tt < tokens && k < a.channels;
+            const int64_t row = row0 + base + tt;
+            sx[j] = ok ? x[row * a.x_stride + k] : zero;
+            sd[j] = ok ? dt_raw[row * a.dt_stride + k] : zero;
+            sz[j] = (ok && z) ? z[row * a.z_stride + k] : zero;
+        }
+#pragma unroll
+        for (int j = 0; j < BS; ++j) {
+            const int i = tid + SCAN_THREADS * j;
+            const int tt = i / (2 * NP), col = i % (2 * NP);
+            const int n = col % NP;
+            const bool ok = tt < tokens && tt < CHUNK && n < N;
+            sb[j] = ok ? bc[static_cast<int64_t>(row0 + base + tt) * a.bc_stride + (col < NP ? a.b0 : a.c0) + n] : zero;
         }
     };
-    if (count > 0) fetch(0, xv, dv, zv, Bn, Cn);
-    for (int i = 0; i < count; ++i) {
-        float nx = 0.f, nd = 0.f, nz = 0.f, nB[NS], nC[NS];
-        if (i + 1 < count) fetch(i + 1, nx, nd, nz, nB, nC);
-        const float dt = softplus_f(dv + bias);
-        const float dtx = dt * xv;
-        float part = 0.f;
+    auto stash = [&]() {
 #pragma unroll
-        for (int j = 0; j < NS; ++j) {
-            S[j] = fmaf(expf(dt * A[j]), S[j], dtx * Bn[j]);
-            part = fmaf(S[j], Cn[j], part);
+        for (int j = 0; j < XS; ++j) {
+            const int i = tid + SCAN_THREADS * j;
+            float* r = rows_s + (i / CH) * W + i % CH;
+            r[0] = to_f32<TX>(sx[j]);
+            r[CH] = softplus_f<TX>(to_f32<TX>(sd[j]) + bias_s[i % CH]);
+            r[2 * CH] = z ? silu_f<TX>(to_f32<TX>(sz[j])) : 1.f;
         }
-        for (int off = L / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, PULSE_WAVE);
-        if (live && sub == 0) {
-            float out = fmaf(dsk, xv, part);
-            if (z) out *= silu_f(zv);
-            y[static_cast<int64_t>(row0 + i) * a.y_stride + c] = from_f32<TX>(out);
-        }
-        if (i + 1 < count) {
-            xv = nx; dv = nd; zv = nz;
 #pragma unroll
-            for (int j = 0; j < NS; ++j) { Bn[j] = nB[j]; Cn[j] = nC[j]; }
+        for (int j = 0; j < BS; ++j) {
+            const int i = tid + SCAN_THREADS * j;
+            if (i < CHUNK * 2 * NP) rows_s[(i / (2 * NP)) * W + 3 * CH + i % (2 * NP)] = to_f32<TX>(sb[j]);
         }
+    };
+
+    fetch(0, min(CHUNK, count));
+    __syncthreads();   // bias_s
+    stash();
+    __syncthreads();
+    for (int base = 0; base < count; base += CHUNK) {
+        const int here = min(CHUNK, count - base);
+        const int next = min(CHUNK, count - base - CHUNK);
+        if (next > 0) fetch(base + CHUNK, next);
+#pragma unroll 2
+        for (int tt = 0; tt < here; ++tt) {
+            const float* r = rows_s + tt * W;
+            const float xv = r[ch], dt = r[CH + ch], gate = r[2 * CH + ch];
+            const float dtx = dt * xv;
+            float part = 0.f;
+#pragma unroll
+            for (int j = 0; j < NS; ++j) {
+                S[j] = fmaf(decay_exp<TX>(dt * A[j]), S[j], dtx * r[3 * CH + sub * NS + j]);
+                part = fmaf(S[j], r[3 * CH + NP + sub * NS + j], part);
+            }
+            part = group_sum<L>(part);
+            const float out = fmaf(dsk, xv, part) * gate;
+            if (sub == 0) y_s[tt * CH + ch] = out;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < XS; ++j) {
+            const int i = tid + SCAN_THREADS * j;
+            const int tt = i / CH, k = c0 + i % CH;
+            if (tt < here && k < a.channels)
+                y[static_cast<int64_t>(row0 + base + tt) * a.y_stride + k] = from_f32<TX>(y_s[i]);
+        }
+        if (next > 0) stash();   // (the rows in LDS have been read by everybody: the barrier above)
+        __syncthreads();
     }
     if (live) {
 #pragma unroll
         for (int j = 0; j < NS; ++j) {
-            const int n = sub + L * j;
+            const int n = sub * NS + j;
             if (n < N) srow[n] = S[j];
         }
     }
@@ -188,11 +323,23 @@ extern "C" int pulse_causal_conv(const void* in, int64_t in_stride, int x_dtype,
     a.channels = channels; a.taps = n_taps; a.n_state = n_state; a.state_row = n_state + n_taps - 1;
     a.in_stride = in_stride; a.out_stride = out_stride; a.tokens = tokens; a.entries = entries;
     const int blocks = (channels + 255) / 256;
-    PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(w_dtype, TW,
-        hipLaunchKernelGGL((causal_conv_kernel<TX, TW>), dim3(blocks, tokens), dim3(256), 0, stream,
-                           static_cast<const TX*>(in), static_cast<const TW*>(taps), static_cast<const TW*>(bias),
-                           static_cast<TX*>(out), state, positions, token_entry, entry_start, entry_first_row,
-                           entry_slot, a)));
+    // (few tokens, a decoding step: a thread a channel gives more workgroups, which is what counts there)
+    const bool wide = tokens >= 64 && x_dtype == PULSE_BF16 && channels % 8 == 0 && in_stride % 8 == 0 && out_stride % 8 == 0 &&
+                      reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    if (wide) {
+        const int threads = channels / 8 >= 256 ? 256 : 64;
+        PULSE_DISPATCH_DTYPE(w_dtype, TW,
+            hipLaunchKernelGGL((causal_conv_bf16x8_kernel<TW>), dim3((channels / 8 + threads - 1) / threads, tokens),
+                               dim3(threads), 0, stream, static_cast<const bf16_t*>(in), static_cast<const TW*>(taps),
+                               static_cast<const TW*>(bias), static_cast<bf16_t*>(out), state, positions, token_entry,
+                               entry_start, entry_first_row, entry_slot, a));
+    } else {
+        PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(w_dtype, TW,
+            hipLaunchKernelGGL((causal_conv_kernel<TX, TW>), dim3(blocks, tokens), dim3(256), 0, stream,
+                               static_cast<const TX*>(in), static_cast<const TW*>(taps), static_cast<const TW*>(bias),
+                               static_cast<TX*>(out), state, positions, token_entry, entry_start, entry_first_row,
+                               entry_slot, a)));
+    }
     PULSE_LAUNCH_CHECK("causal_conv");
     if (n_taps > 1) {
         PULSE_DISPATCH_DTYPE(x_dtype, TX,
@@ -221,27 +368,42 @@ extern "C" int pulse_selective_scan(const void* x, int64_t x_stride, const void*
                   "selective_scan: B and C do not lie inside their rows");
     PULSE_REQUIRE(entries < 65536, "selective_scan: at most 65535 entries a step");
     if (entries == 0) return 0;
-    int lanes = 1;
-    while (lanes < 16 && lanes < n_state) lanes *= 2;
+    // lanes a channel: few while a lane's share of the states stays within 16 (see the kernel); more where that
+    // would leave compute units without a workgroup (one long prompt: then the walk's latency is what counts, and
+    // a channel's states spread over more lanes shorten it)
+    int lanes = n_state == 1 ? 1 : (n_state == 2 ? 2 : (n_state <= 64 ? 4 : 16));
+    const int64_t units = pulse_compute_units();
+    if (lanes == 4 && n_state >= 8 && static_cast<int64_t>((channels + 63) / 64) * entries < units) lanes = 8;
+    if (lanes == 8 && n_state >= 16 && static_cast<int64_t>((channels + 31) / 32) * entries < units) lanes = 16;
+    if (lanes == 8 && n_state > 128) lanes = 16;
     const int ns = (n_state + lanes - 1) / lanes;
     ScanArgs a;
-    a.channels = channels; a.n_state = n_state; a.state_row = state_row; a.lanes = lanes; a.entries = entries;
+    a.channels = channels; a.n_state = n_state; a.state_row = state_row; a.entries = entries;
     a.x_stride = x_stride; a.dt_stride = dt_stride; a.bc_stride = bc_stride; a.z_stride = z_stride; a.y_stride = y_stride;
     a.b0 = b0; a.c0 = c0;
-    const int per_block = 256 / lanes;
+    const int per_block = SCAN_THREADS / lanes;
     const dim3 grid((channels + per_block - 1) / per_block, entries);
-#define PULSE_SCAN(NS_)                                                                                              \
+#define PULSE_SCAN(NS_, L_)                                                                                          \
     PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(w_dtype, TW,                                              \
-        hipLaunchKernelGGL((selective_scan_kernel<TX, TW, NS_>), grid, dim3(256), 0, stream,                        \
+        hipLaunchKernelGGL((selective_scan_kernel<TX, TW, NS_, L_>), grid, dim3(SCAN_THREADS), 0, stream,           \
                            static_cast<const TX*>(x), static_cast<const TX*>(dt_raw), static_cast<const TW*>(dt_bias), \
                            static_cast<const TW*>(a_log), static_cast<const TX*>(bc), static_cast<const TW*>(d_skip), \
                            static_cast<const TX*>(z), static_cast<TX*>(y), state, entry_start, entry_first_row,       \
                            entry_slot, a)))
-    if (ns <= 1) PULSE_SCAN(1);
-    else if (ns <= 2) PULSE_SCAN(2);
-    else if (ns <= 4) PULSE_SCAN(4);
-    else if (ns <= 8) PULSE_SCAN(8);
-    else PULSE_SCAN(16);
+#define PULSE_SCAN_NS(L_)                        \
+    do {                                         \
+        if (ns <= 1) PULSE_SCAN(1, L_);          \
+        else if (ns <= 2) PULSE_SCAN(2, L_);     \
+        else if (ns <= 4) PULSE_SCAN(4, L_);     \
+        else if (ns <= 8) PULSE_SCAN(8, L_);     \
+        else PULSE_SCAN(16, L_);                 \
+    } while (0)
+    if (lanes == 1) PULSE_SCAN(1, 1);
+    else if (lanes == 2) PULSE_SCAN(1, 2);
+    else if (lanes == 4) PULSE_SCAN_NS(4);
+    else if (lanes == 8) PULSE_SCAN_NS(8);
+    else PULSE_SCAN_NS(16);
+#undef PULSE_SCAN_NS
 #undef PULSE_SCAN
     PULSE_LAUNCH_CHECK("selective_scan");
     return 0;

@@ -31,51 +31,64 @@ struct StreamArgs {
     int has_out;     // step 2 is wanted
 };
 
-template <typename TYIN, typename TW, typename TO>
-__global__ __launch_bounds__(256) void streams_step_kernel(float* __restrict__ x, const TYIN* __restrict__ y,
-                                                           const float* __restrict__ mix,
-                                                           const float* __restrict__ out_w,
-                                                           const float* __restrict__ in_w,
-                                                           const int* __restrict__ rows, const TW* __restrict__ w,
-                                                           const TW* __restrict__ b, TO* __restrict__ out,
-                                                           StreamArgs a) {
+// SC: the number of streams where it is one the kernel is compiled for (1 to 4: loops unroll, the mixing matrix
+// lies in registers), 0: any number up to MAX_STREAMS, read from the arguments.
+template <typename TYIN, typename TW, typename TO, int SC>
+__global__ __launch_bounds__(1024) void streams_step_kernel(float* __restrict__ x, const TYIN* __restrict__ y,
+                                                            const float* __restrict__ mix,
+                                                            const float* __restrict__ out_w,
+                                                            const float* __restrict__ in_w,
+                                                            const int* __restrict__ rows, const TW* __restrict__ w,
+                                                            const TW* __restrict__ b, TO* __restrict__ out,
+                                                            StreamArgs a) {
     extern __shared__ float u_s[];    // [hidden]
     __shared__ float scratch[16];
     __shared__ float mix_s[MAX_STREAMS * MAX_STREAMS], ow_s[MAX_STREAMS], iw_s[MAX_STREAMS];
+    constexpr int MS = SC ? SC : MAX_STREAMS;
     const int r = blockIdx.x;
     const int64_t t = rows ? rows[r] : r;
-    const int S = a.streams, H = a.hidden;
+    const int S = SC ? SC : a.streams, H = a.hidden;
     if (threadIdx.x < S * S && mix) mix_s[threadIdx.x] = mix[threadIdx.x];
     if (threadIdx.x < S) {
         ow_s[threadIdx.x] = out_w ? out_w[threadIdx.x] : 0.f;
         iw_s[threadIdx.x] = in_w ? in_w[threadIdx.x] : 1.f;
     }
     __syncthreads();
+    float mixr[SC ? SC * SC : 1], owr[MS], iwr[MS];
+#pragma unroll
+    for (int s = 0; s < MS; ++s) {
+        owr[s] = s < S ? ow_s[s] : 0.f;
+        iwr[s] = s < S ? iw_s[s] : 0.f;
+    }
+    if constexpr (SC > 0) {
+#pragma unroll
+        for (int i = 0; i < SC * SC; ++i) mixr[i] = y ? mix_s[i] : 0.f;
+    }
     float* xrow = x + t * S * H;
     float sum = 0.f;
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
-        float old[MAX_STREAMS];
+        float old[MS];
 #pragma unroll
-        for (int s = 0; s < MAX_STREAMS; ++s) old[s] = s < S ? xrow[s * H + i] : 0.f;
+        for (int s = 0; s < MS; ++s) old[s] = s < S ? xrow[s * H + i] : 0.f;
         float u = 0.f;
         if (y) {
             const float yv = to_f32<TYIN>(y[t * H + i]);
 #pragma unroll
-            for (int to = 0; to < MAX_STREAMS; ++to) {
+            for (int to = 0; to < MS; ++to) {
                 if (to < S) {
                     float v = 0.f;
 #pragma unroll
-                    for (int s = 0; s < MAX_STREAMS; ++s)
-                        if (s < S) v = fmaf(mix_s[s * S + to], old[s], v);
-                    v = fmaf(ow_s[to], yv, v);
+                    for (int s = 0; s < MS; ++s)
+                        if (s < S) v = fmaf(SC ? mixr[SC ? s * SC + to : 0] : mix_s[s * S + to], old[s], v);
+                    v = fmaf(owr[to], yv, v);
                     xrow[to * H + i] = v;
-                    u = fmaf(iw_s[to], v, u);
+                    u = fmaf(iwr[to], v, u);
                 }
             }
         } else {
 #pragma unroll
-            for (int s = 0; s < MAX_STREAMS; ++s)
-                if (s < S) u = fmaf(iw_s[s], old[s], u);
+            for (int s = 0; s < MS; ++s)
+                if (s < S) u = fmaf(iwr[s], old[s], u);
         }
         if (a.has_out) {
             u_s[i] = u;
@@ -135,10 +148,19 @@ extern "C" int pulse_streams_step(float* x, int tokens, int streams, int hidden,
     if (n_rows == 0) return 0;
     StreamArgs a;
     a.streams = streams; a.hidden = hidden; a.kind = kind; a.eps = eps; a.has_out = out ? 1 : 0;
-    PULSE_DISPATCH_DTYPE(y_dtype, TYIN, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(out_dtype, TO,
-        hipLaunchKernelGGL((streams_step_kernel<TYIN, TW, TO>), dim3(n_rows), dim3(256), lds, stream, x,
-                           static_cast<const TYIN*>(y), mix, out_w, in_w, rows, static_cast<const TW*>(w),
-                           static_cast<const TW*>(b), static_cast<TO*>(out), a))));
+    // few rows of a wide residual (a decoding step): wider workgroups, since there are not many of them
+    const int threads = (n_rows <= 256 && hidden >= 2048) ? 1024 : 256;
+#define PULSE_STREAMS(SC_)                                                                                           \
+    PULSE_DISPATCH_DTYPE(y_dtype, TYIN, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(out_dtype, TO,        \
+        hipLaunchKernelGGL((streams_step_kernel<TYIN, TW, TO, SC_>), dim3(n_rows), dim3(threads), lds, stream, x,    \
+                           static_cast<const TYIN*>(y), mix, out_w, in_w, rows, static_cast<const TW*>(w),           \
+                           static_cast<const TW*>(b), static_cast<TO*>(out), a))))
+    if (streams == 1) PULSE_STREAMS(1);
+    else if (streams == 2) PULSE_STREAMS(2);
+    else if (streams == 3) PULSE_STREAMS(3);
+    else if (streams == 4) PULSE_STREAMS(4);
+    else PULSE_STREAMS(0);
+#undef PULSE_STREAMS
     PULSE_LAUNCH_CHECK("streams_step");
     return 0;
 }

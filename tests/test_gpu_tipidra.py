@@ -222,7 +222,7 @@ def test_streams_their_update_and_the_layer_norm(dtype, streams, hidden):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("inner,state,taps", [(80, 5, 2), (128, 16, 4), (48, 24, 3), (200, 32, 4), (33, 70, 1),
-                                              (64, 1, 4)])
+                                              (64, 1, 4), (72, 2, 4), (40, 3, 2), (2048, 16, 4), (24, 256, 3)])
 def test_the_convolution_and_the_recurrence(dtype, inner, state, taps):
     """Three requests in one step (a portion of 37 tokens that continues a state, a fresh prompt of 20 in a slot that
     holds NaN, a single decoded token), then the same requests a few tokens further (fewer than the taps for one of
