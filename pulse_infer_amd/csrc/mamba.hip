@@ -74,7 +74,10 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const TX* __restrict__
     out[static_cast<int64_t>(t) * a.out_stride + c] = from_f32<TX>(silu_f<TX>(acc));
 }
 
-// The same for bfloat16 rows whose sizes allow 16-byte accesses: a thread takes 8 neighbouring channels of a token.
+// The same for bfloat16 rows whose sizes allow 16-byte accesses and at most 8 taps: a thread takes 8 neighbouring
+// channels of CONV_TOKENS consecutive tokens, with the channels' taps in registers.
+constexpr int CONV_TOKENS = 8;
+
 template <typename TW>
 __global__ __launch_bounds__(256) void causal_conv_bf16x8_kernel(const bf16_t* __restrict__ in, const TW* __restrict__ taps,
                                                                  const TW* __restrict__ bias, bf16_t* __restrict__ out,
@@ -85,42 +88,49 @@ __global__ __launch_bounds__(256) void causal_conv_bf16x8_kernel(const bf16_t* _
                                                                  const int* __restrict__ entry_first_row,
                                                                  const int* __restrict__ entry_slot, ConvArgs a) {
     const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
-    const int t = blockIdx.y;
     if (c >= a.channels) return;
-    const int e = token_entry[t];
-    const int start = entry_start[e], row0 = entry_first_row[e];
-    const int pos = positions[t];
     const int K = a.taps;
-    const float* tail = state + (static_cast<int64_t>(entry_slot[e]) * a.channels + c) * a.state_row + a.n_state;
-    float acc[8];
+    float w[8][8], b[8];   // [tap][channel]
 #pragma unroll
-    for (int u = 0; u < 8; ++u) acc[u] = bias ? to_f32<TW>(bias[c + u]) : 0.f;
-    for (int j = 0; j < K; ++j) {
-        const int q = pos - (K - 1) + j;
-        float v[8];
-        if (q >= start) {
-            const pulse_i32x4 raw = *reinterpret_cast<const pulse_i32x4*>(in + static_cast<int64_t>(row0 + q - start) * a.in_stride + c);
+    for (int u = 0; u < 8; ++u) {
+        b[u] = bias ? to_f32<TW>(bias[c + u]) : 0.f;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const uint32_t two = static_cast<uint32_t>(raw[u]);
-                v[2 * u] = __uint_as_float(two << 16);
-                v[2 * u + 1] = __uint_as_float(two & 0xffff0000u);
-            }
-        } else if (q >= 0) {
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = tail[static_cast<int64_t>(u) * a.state_row + (K - 1) - (start - q)];
-        } else {
-            continue;
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) acc[u] = fmaf(to_f32<TW>(taps[static_cast<int64_t>(c + u) * K + j]), v[u], acc[u]);
+        for (int j = 0; j < 8; ++j) w[j][u] = j < K ? to_f32<TW>(taps[static_cast<int64_t>(c + u) * K + j]) : 0.f;
     }
-    uint32_t packed[4];
+    const int t_end = min(a.tokens, static_cast<int>(blockIdx.y + 1) * CONV_TOKENS);
+    for (int t = blockIdx.y * CONV_TOKENS; t < t_end; ++t) {
+        const int e = token_entry[t];
+        const int start = entry_start[e], row0 = entry_first_row[e];
+        const int pos = positions[t];
+        const float* tail = state + (static_cast<int64_t>(entry_slot[e]) * a.channels + c) * a.state_row + a.n_state;
+        float acc[8];
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
-        packed[u] = static_cast<uint32_t>(f32_to_bf16(silu_f<bf16_t>(acc[2 * u]))) |
-                    (static_cast<uint32_t>(f32_to_bf16(silu_f<bf16_t>(acc[2 * u + 1]))) << 16);
-    *reinterpret_cast<uint4*>(out + static_cast<int64_t>(t) * a.out_stride + c) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+        for (int u = 0; u < 8; ++u) acc[u] = b[u];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (j >= K) continue;
+            const int q = pos - (K - 1) + j;
+            if (q >= start) {
+                const pulse_i32x4 raw = *reinterpret_cast<const pulse_i32x4*>(in + static_cast<int64_t>(row0 + q - start) * a.in_stride + c);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t two = static_cast<uint32_t>(raw[u]);
+                    acc[2 * u] = fmaf(w[j][2 * u], __uint_as_float(two << 16), acc[2 * u]);
+                    acc[2 * u + 1] = fmaf(w[j][2 * u + 1], __uint_as_float(two & 0xffff0000u), acc[2 * u + 1]);
+                }
+            } else if (q >= 0) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    acc[u] = fmaf(w[j][u], tail[static_cast<int64_t>(u) * a.state_row + (K - 1) - (start - q)], acc[u]);
+            }
+        }
+        uint32_t packed[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            packed[u] = static_cast<uint32_t>(f32_to_bf16(silu_f<bf16_t>(acc[2 * u]))) |
+                        (static_cast<uint32_t>(f32_to_bf16(silu_f<bf16_t>(acc[2 * u + 1]))) << 16);
+        *reinterpret_cast<uint4*>(out + static_cast<int64_t>(t) * a.out_stride + c) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    }
 }
 
 template <typename TX>
@@ -269,7 +279,6 @@ __global__ __launch_bounds__(SCAN_THREADS) void selective_scan_kernel(
         const int here = min(CHUNK, count - base);
         const int next = min(CHUNK, count - base - CHUNK);
         if (next > 0) fetch(base + CHUNK, next);
-#pragma unroll 2
         for (int tt = 0; tt < here; ++tt) {
             const float* r = rows_s + tt * W;
             const float xv = r[ch], dt = r[CH + ch], gate = r[2 * CH + ch];
@@ -324,12 +333,13 @@ extern "C" int pulse_causal_conv(const void* in, int64_t in_stride, int x_dtype,
     a.in_stride = in_stride; a.out_stride = out_stride; a.tokens = tokens; a.entries = entries;
     const int blocks = (channels + 255) / 256;
     // (few tokens, a decoding step: a thread a channel gives more workgroups, which is what counts there)
-    const bool wide = tokens >= 64 && x_dtype == PULSE_BF16 && channels % 8 == 0 && in_stride % 8 == 0 && out_stride % 8 == 0 &&
+    const bool wide = tokens >= 64 && n_taps <= 8 && x_dtype == PULSE_BF16 && channels % 8 == 0 && in_stride % 8 == 0 && out_stride % 8 == 0 &&
                       reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
     if (wide) {
         const int threads = channels / 8 >= 256 ? 256 : 64;
         PULSE_DISPATCH_DTYPE(w_dtype, TW,
-            hipLaunchKernelGGL((causal_conv_bf16x8_kernel<TW>), dim3((channels / 8 + threads - 1) / threads, tokens),
+            hipLaunchKernelGGL((causal_conv_bf16x8_kernel<TW>),
+                               dim3((channels / 8 + threads - 1) / threads, (tokens + CONV_TOKENS - 1) / CONV_TOKENS),
                                dim3(threads), 0, stream, static_cast<const bf16_t*>(in), static_cast<const TW*>(taps),
                                static_cast<const TW*>(bias), static_cast<bf16_t*>(out), state, positions, token_entry,
                                entry_start, entry_first_row, entry_slot, a));
