@@ -260,7 +260,7 @@ def tipidra_layers(size, layers):
     experts; the state-space mixer with a dense feed-forward.  The routed feed-forward has 16 experts an eighth as
     wide as the dense one, 4 chosen a token: half of the dense feed-forward's arithmetic a token."""
     attention = {"dim": size["dim"], "heads": size["heads"], "kv_heads": size["kv_heads"], "vdim": size["dim"],
-                 "rot": {"base": 1e6, "dims": size["dim"] // 2}, "scale": size["dim"] ** -0.5, "softcap": 50.0}
+                 "rot": {"base": 1e6, "dims": size["dim"] // 2}, "scale": size["dim"] ** -0.5, "softcap": 30.0}
     ssm = {"inner": 2 * size["width"], "state": 16, "dt_rank": size["width"] // 16, "conv": 4}
     dense = {"ff": size["ff"], "kind": "dense"}
     routed = {"expert": {"ff": size["ff"] // 8, "limit": 7.0}, "kind": "moe", "router": {"experts": 16, "top": 4}}

@@ -4,10 +4,11 @@
     llm = LLM.from_pretrained("model_dir", dtype="bfloat16")
     out = llm.generate([[1, 2, 3]], max_new_tokens=16)
 """
-from .config import ConfigError, DirozenConfig, KesovikConfig, Qwen3Config, load_config, register_architecture
+from .config import (ConfigError, DirozenConfig, KesovikConfig, Qwen3Config, TipidraConfig, load_config,
+                     register_architecture)
 from .sampling.params import SamplingParams
 
-__all__ = ["ConfigError", "DirozenConfig", "KesovikConfig", "Qwen3Config", "load_config", "register_architecture", "SamplingParams", "LLM",
+__all__ = ["ConfigError", "DirozenConfig", "KesovikConfig", "Qwen3Config", "TipidraConfig", "load_config", "register_architecture", "SamplingParams", "LLM",
            "ContinuousBatchEngine"]
 
 

@@ -7,7 +7,8 @@
 //     x_t'   = sum_s mix[s, t] x_s + out[t] * y                   (all streams at once from the old ones)
 //
 // pulse_streams_step does, for every row r (token s = rows ? rows[r] : r), whichever of these it is handed:
-//   1. the update of the token's streams with a sublayer's result y (written back in place), then
+//   1. the update of the token's streams with a sublayer's result y (written back in place; with a list of rows
+//      the new streams are formed but not stored: whoever gathers rows reads the residual for the last time), then
 //   2. u = sum_s in[s] x_s over the (new) streams (in == null: every factor is one), and the norm of u:
 //        layer norm  (u - mean) / sqrt(var + eps) * w + b    (var the mean of the squared deviations), or
 //        RMS norm    u / sqrt(mean(u^2) + eps) * w           (b == null and kind == 1)
@@ -81,7 +82,7 @@ __global__ __launch_bounds__(1024) void streams_step_kernel(float* __restrict__ 
                     for (int s = 0; s < MS; ++s)
                         if (s < S) v = fmaf(SC ? mixr[SC ? s * SC + to : 0] : mix_s[s * S + to], old[s], v);
                     v = fmaf(owr[to], yv, v);
-                    xrow[to * H + i] = v;
+                    if (!rows) xrow[to * H + i] = v;
                     u = fmaf(iwr[to], v, u);
                 }
             }
@@ -138,7 +139,7 @@ extern "C" int pulse_streams_step(float* x, int tokens, int streams, int hidden,
     PULSE_REQUIRE(streams >= 1 && streams <= MAX_STREAMS, "streams_step: 1 to %d streams, got %d", MAX_STREAMS, streams);
     PULSE_REQUIRE(pulse_dtype_ok(y_dtype) && pulse_dtype_ok(w_dtype) && pulse_dtype_ok(out_dtype), "streams_step: bad dtype tag");
     PULSE_REQUIRE(!y || (mix && out_w), "streams_step: an update needs the mixing matrix and the result's factors");
-    PULSE_REQUIRE(!(y && rows), "streams_step: an update runs over all rows, not gathered ones");
+    PULSE_REQUIRE(!(y && rows) || out, "streams_step: an update of gathered rows is not stored, so it comes with a norm");
     PULSE_REQUIRE(y || out, "streams_step: nothing to do");
     PULSE_REQUIRE(!out || w, "streams_step: the norm's weight is missing");
     PULSE_REQUIRE(kind == 0 || kind == 1, "streams_step: unknown norm %d", kind);

@@ -1017,7 +1017,8 @@ def streams_step(x: torch.Tensor, streams: int, update: Optional[tuple] = None, 
     ``update`` = (y [T, H], mix float32 [streams, streams] indexed [from, to], out_factors float32 [streams]):
     x_t <- sum_s mix[s, t] x_s + out_factors[t] * y, all streams at once, written back.  ``norm`` = (kind, weight,
     bias or None, eps) with ``out`` [rows, H]: u = sum_s in_weight[s] x_s (None: the plain sum) over the new streams,
-    normed (kind "layernorm" or "rmsnorm") and rounded once; ``rows`` gathers (without an update only)."""
+    normed (kind "layernorm" or "rmsnorm") and rounded once; ``rows`` gathers, and an update of gathered rows is
+    formed but not written back (the residual is then read for the last time)."""
     _gpu("streams_step", x, in_weight, out, rows)
     _need(1 <= streams <= MAX_STREAMS, f"streams_step: 1 to {MAX_STREAMS} streams, got {streams}")
     _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and x.shape[1] % streams == 0,
@@ -1027,7 +1028,7 @@ def streams_step(x: torch.Tensor, streams: int, update: Optional[tuple] = None, 
     if update is not None:
         y, mix, out_w = update
         _gpu("streams_step", y, mix, out_w)
-        _need(rows is None, "streams_step: an update runs over all rows")
+        _need(rows is None or norm is not None, "streams_step: an update of gathered rows comes with a norm")
         _need(y.is_contiguous() and tuple(y.shape) == (tokens, hidden), f"streams_step: y must be [{tokens}, {hidden}]")
         _need(mix.dtype == torch.float32 and mix.is_contiguous() and tuple(mix.shape) == (streams, streams)
               and out_w.dtype == torch.float32 and out_w.is_contiguous() and out_w.numel() == streams,

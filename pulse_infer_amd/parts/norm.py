@@ -84,13 +84,11 @@ class LayerNorm(Part):
     def apply(self, h: torch.Tensor, delta: Any, out: torch.Tensor, rows: Optional[torch.Tensor] = None,
               stream_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
         """out = norm(sum_s weights[s] * h_s) after ``delta`` has gone into h: a ``StreamUpdate`` (done by the same
-        kernel), a tensor of h's shape (added first), or None."""
+        kernel; with gathered rows the updated streams are used but not stored: who gathers rows reads the residual
+        for the last time), a tensor of h's shape (added first), or None."""
         update = None
         if isinstance(delta, StreamUpdate):
-            if rows is None:
-                update = (delta.y, delta.mix, delta.out)
-            else:
-                delta.apply_to(h)
+            update = (delta.y, delta.mix, delta.out)
         elif delta is not None:
             kernels.residual_add(h, delta)
         kernels.streams_step(h, self.streams, update=update, in_weight=stream_weights,
