@@ -252,10 +252,11 @@ class CacheManager:
                 continue
             table = g.tables[request]
             dead = min(g.first_needed_token(computed) // g.page_size, len(table))
-            gone = [table[i] for i in range(dead) if table[i] >= 0]
+            kept = g.pages_for(int(getattr(g.spec, "keep_first", 0) or 0))   # pages of the first tokens stay
+            gone = [table[i] for i in range(kept, dead) if table[i] >= 0]
             if gone:
                 g.pool.release(gone)
-                for i in range(dead):
+                for i in range(kept, dead):
                     table[i] = -1
                 req.stamp = self._tick()
 

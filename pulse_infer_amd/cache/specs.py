@@ -8,7 +8,9 @@ A spec is a small hashable object that the cache manager asks, never inspects:
   request's slot.
 * ``window`` (per-token specs) — None: every token is kept; n: only the last n
   tokens are ever read, so pages wholly below the window go back to the pool
-  while the request still runs.
+  while the request still runs.  ``keep_first`` (optional, default 0): the first
+  tokens of a request that stay readable whatever the window; the pages that hold
+  them are kept.
 * ``bytes_per_token(element_size)`` (per-token specs) — what one token costs one
   run, for sizing pools and pricing steps.
 * ``allocate(runs, units, page_size, device, dtype)`` — the storage of all runs of
@@ -64,6 +66,7 @@ class PagedKVSpec:
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None  # None: all keys
+    keep_first: int = 0           # with a window: the first tokens stay readable, so their pages are never given back
 
     per_token = True
 

@@ -41,7 +41,7 @@ extern "C" int pulse_embed_gather(const int* ids, const void* table, int table_d
 
 // --------------------------------------------------- residual add + RMSNorm
 // For output row r (input row s = rows ? rows[r] : r):
-//   v = h[s] + delta[s]            (delta optional)
+//   v = h[s] + dscale * delta[s]   (delta optional; dscale: a factor on the update, 1 for the plain sum)
 //   h[s] = v                       (only when write_back)
 //   y[r] = v * (1 / sqrt(mean(v^2) + eps)) * (w_offset + w)      one rounding at the end
 // (w_offset: 0 for a weight stored as the factor itself, 1 for a weight stored as the factor's distance from one)
@@ -50,7 +50,8 @@ extern "C" int pulse_embed_gather(const int* ids, const void* table, int table_d
 template <typename TD, typename TW, typename TY>
 __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, int parts, int64_t part_stride,
                                    const int* __restrict__ rows, const TW* __restrict__ w,
-                                   TY* __restrict__ y, int hidden, float eps, int write_back, float w_offset) {
+                                   TY* __restrict__ y, int hidden, float eps, int write_back, float w_offset,
+                                   float dscale) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const int64_t s = rows ? rows[r] : r;
@@ -60,7 +61,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = hrow[i];
         if (drow)
-            for (int p = 0; p < parts; ++p) v += to_f32<TD>(drow[p * part_stride + i]);
+            for (int p = 0; p < parts; ++p) v += dscale * to_f32<TD>(drow[p * part_stride + i]);
         ss += v * v;
     }
     ss = block_sum(ss, scratch);
@@ -69,7 +70,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = hrow[i];
         if (drow)
-            for (int p = 0; p < parts; ++p) v += to_f32<TD>(drow[p * part_stride + i]);
+            for (int p = 0; p < parts; ++p) v += dscale * to_f32<TD>(drow[p * part_stride + i]);
         if (write_back) hrow[i] = v;
         yrow[i] = from_f32<TY>(v * inv * (w_offset + to_f32<TW>(w[i])));
     }
@@ -100,7 +101,8 @@ template <typename TD, typename TW, typename TY, int THREADS, bool PARTS>
 __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                                               int parts, int64_t part_stride,
                                                               const int* __restrict__ rows, const TW* __restrict__ w,
-                                                              TY* __restrict__ y, int hidden, float eps, int write_back, float w_offset) {
+                                                              TY* __restrict__ y, int hidden, float eps, int write_back, float w_offset,
+                                                              float dscale) {
     __shared__ float scratch[16];
     typedef typename Vec4<TD>::type VD;
     typedef typename Vec4<TW>::type VW;
@@ -121,7 +123,7 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
                 v[c] = hrow[i];
                 if (drow) {
                     const float4 d = widen4(drow[i]);
-                    v[c].x += d.x; v[c].y += d.y; v[c].z += d.z; v[c].w += d.w;
+                    v[c].x += dscale * d.x; v[c].y += dscale * d.y; v[c].z += dscale * d.z; v[c].w += dscale * d.w;
                 }
                 ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
             }
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
 #pragma unroll
             for (int c = 0; c < CHUNKS; ++c) {
                 const int i = threadIdx.x + c * THREADS;
-                if (i < nvec) { v[c].x += d[c].x; v[c].y += d[c].y; v[c].z += d[c].z; v[c].w += d[c].w; }
+                if (i < nvec) { v[c].x += dscale * d[c].x; v[c].y += dscale * d[c].y; v[c].z += dscale * d[c].z; v[c].w += dscale * d[c].w; }
             }
         }
 #pragma unroll
@@ -175,7 +177,8 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
 // order, is what is normalised (the shares of a product whose inner dimension was split).
 extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, int parts, int64_t part_stride,
                                  const int* rows, const void* w, int w_dtype, void* y, int y_dtype, int out_rows,
-                                 int hidden, float eps, int write_back, float w_offset, hipStream_t stream) {
+                                 int hidden, float eps, int write_back, float w_offset, float dscale,
+                                 hipStream_t stream) {
     PULSE_REQUIRE(parts >= 1 && (parts == 1 || (delta && part_stride % 4 == 0)), "add_rmsnorm: bad parts of the update");
     PULSE_REQUIRE(out_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d H=%d", out_rows, hidden);
     PULSE_REQUIRE(pulse_dtype_ok(delta_dtype) && pulse_dtype_ok(w_dtype) && pulse_dtype_ok(y_dtype),
@@ -190,20 +193,20 @@ extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, i
             if (parts > 1)
                 hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 1024, true>), dim3(out_rows), dim3(1024), 0, stream, h,
                                    static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
-                                   static_cast<TY*>(y), hidden, eps, write_back, w_offset);
+                                   static_cast<TY*>(y), hidden, eps, write_back, w_offset, dscale);
             else if (out_rows <= 256 && hidden >= 2048)   // few rows: bound by round trips, not by bandwidth
                 hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 1024, false>), dim3(out_rows), dim3(1024), 0, stream, h,
                                    static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
-                                   static_cast<TY*>(y), hidden, eps, write_back, w_offset);
+                                   static_cast<TY*>(y), hidden, eps, write_back, w_offset, dscale);
             else
                 hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 256, false>), dim3(out_rows), dim3(256), 0, stream, h,
                                    static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
-                                   static_cast<TY*>(y), hidden, eps, write_back, w_offset))));
+                                   static_cast<TY*>(y), hidden, eps, write_back, w_offset, dscale))));
     } else {
         PULSE_DISPATCH_DTYPE(delta_dtype, TD, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(y_dtype, TY,
             hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, TY>), dim3(out_rows), dim3(256), 0, stream, h,
                                static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
-                               static_cast<TY*>(y), hidden, eps, write_back, w_offset))));
+                               static_cast<TY*>(y), hidden, eps, write_back, w_offset, dscale))));
     }
     PULSE_LAUNCH_CHECK("add_rmsnorm");
     return 0;
@@ -212,24 +215,47 @@ extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, i
 // -------------------------------------------------------------- residual add
 // h += delta (used where no norm follows).
 template <typename TD>
-__global__ void residual_add_kernel(float* __restrict__ h, const TD* __restrict__ delta, int parts, int64_t n) {
+__global__ void residual_add_kernel(float* __restrict__ h, const TD* __restrict__ delta, int parts, int64_t n,
+                                    float dscale) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= n) return;
     float v = h[i];
-    for (int p = 0; p < parts; ++p) v += to_f32<TD>(delta[p * n + i]);
+    for (int p = 0; p < parts; ++p) v += dscale * to_f32<TD>(delta[p * n + i]);
     h[i] = v;
 }
 
+// h[t, :] += row[:] for every row t of h (a vector added to all tokens of a step).
+template <typename TD>
+__global__ void residual_add_row_kernel(float* __restrict__ h, const TD* __restrict__ row, int64_t n, int hidden) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    h[i] += to_f32<TD>(row[i % hidden]);
+}
+
 // delta holds `parts` (>= 1) arrays of n values one after the other; they are added in order.
-extern "C" int pulse_residual_add(float* h, const void* delta, int delta_dtype, int parts, int64_t n, hipStream_t stream) {
+extern "C" int pulse_residual_add(float* h, const void* delta, int delta_dtype, int parts, int64_t n, float dscale,
+                                  hipStream_t stream) {
     PULSE_REQUIRE(n >= 0 && parts >= 1 && pulse_dtype_ok(delta_dtype) && h && delta, "residual_add: bad arguments");
     if (n == 0) return 0;
     const int64_t blocks = (n + 255) / 256;
     PULSE_REQUIRE(blocks < (1ll << 31), "residual_add: too many elements (%lld)", static_cast<long long>(n));
     PULSE_DISPATCH_DTYPE(delta_dtype, TD,
         hipLaunchKernelGGL(residual_add_kernel<TD>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, h,
-                           static_cast<const TD*>(delta), parts, n));
+                           static_cast<const TD*>(delta), parts, n, dscale));
     PULSE_LAUNCH_CHECK("residual_add");
+    return 0;
+}
+
+extern "C" int pulse_residual_add_row(float* h, const void* row, int row_dtype, int64_t n, int hidden, hipStream_t stream) {
+    PULSE_REQUIRE(n >= 0 && hidden > 0 && n % hidden == 0 && pulse_dtype_ok(row_dtype) && h && row,
+                  "residual_add_row: bad arguments");
+    if (n == 0) return 0;
+    const int64_t blocks = (n + 255) / 256;
+    PULSE_REQUIRE(blocks < (1ll << 31), "residual_add_row: too many elements (%lld)", static_cast<long long>(n));
+    PULSE_DISPATCH_DTYPE(row_dtype, TD,
+        hipLaunchKernelGGL(residual_add_row_kernel<TD>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, h,
+                           static_cast<const TD*>(row), n, hidden));
+    PULSE_LAUNCH_CHECK("residual_add_row");
     return 0;
 }
 

@@ -287,3 +287,37 @@ extern "C" int pulse_moe_down(const void* x, const void* act, int x_dtype, const
     PULSE_LAUNCH_CHECK("moe_down");
     return 0;
 }
+
+// ------------------------------------------------------- a gate of one number a token
+// acc[t, :] += sigmoid(w . x[t]) * y[t, :]: an always-on expert's result y enters the float32 sum of the routed ones
+// times a gate of its own, one number a token, whose logit is a product with the expert's input (float32 inside).
+namespace {
+
+template <typename TX, typename TW>
+__global__ void token_gate_add_kernel(const TX* __restrict__ x, const TW* __restrict__ w, const TX* __restrict__ y,
+                                      float* __restrict__ acc, int hidden) {
+    __shared__ float scratch[16];
+    const int64_t t = blockIdx.x;
+    const TX* xr = x + t * hidden;
+    float dot = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dot = fmaf(to_f32<TX>(xr[i]), to_f32<TW>(w[i]), dot);
+    dot = block_sum(dot, scratch);
+    const float g = 1.0f / (1.0f + expf(-dot));
+    const TX* yr = y + t * hidden;
+    float* ar = acc + t * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) ar[i] = fmaf(g, to_f32<TX>(yr[i]), ar[i]);
+}
+
+}  // namespace
+
+extern "C" int pulse_token_gate_add(const void* x, const void* w, int w_dtype, const void* y, int x_dtype, float* acc,
+                                    int tokens, int hidden, hipStream_t stream) {
+    PULSE_REQUIRE(tokens >= 0 && hidden > 0 && x && w && y && acc && pulse_dtype_ok(w_dtype) && pulse_dtype_ok(x_dtype),
+                  "token_gate_add: bad arguments");
+    if (tokens == 0) return 0;
+    PULSE_DISPATCH_DTYPE(x_dtype, TX, PULSE_DISPATCH_DTYPE(w_dtype, TW,
+        hipLaunchKernelGGL((token_gate_add_kernel<TX, TW>), dim3(tokens), dim3(256), 0, stream, static_cast<const TX*>(x),
+                           static_cast<const TW*>(w), static_cast<const TX*>(y), acc, hidden)));
+    PULSE_LAUNCH_CHECK("token_gate_add");
+    return 0;
+}

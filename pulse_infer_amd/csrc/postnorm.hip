@@ -118,3 +118,34 @@ extern "C" int pulse_round_rows(const float* x, void* y, int y_dtype, int64_t n,
     PULSE_LAUNCH_CHECK("round_rows");
     return 0;
 }
+
+// ---------------------------------------------------------------- xIELU
+// y = a z^2 + z / 2 for z > 0, else b (exp(z) - 1 - z) + z / 2, with a = softplus(p), b = 1/2 + softplus(q) and the two
+// learned numbers p, q read on the device.
+namespace {
+
+__device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+
+template <typename T, typename TP>
+__global__ void xielu_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, const TP* __restrict__ pq) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float a = softplus_f(to_f32<TP>(pq[0])), b = 0.5f + softplus_f(to_f32<TP>(pq[1]));
+    const float z = to_f32<T>(x[i]);
+    const float v = z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z);
+    y[i] = from_f32<T>(v);
+}
+
+}  // namespace
+
+extern "C" int pulse_xielu(const void* x, void* y, int dtype, int64_t n, const void* pq, int pq_dtype, hipStream_t stream) {
+    PULSE_REQUIRE(n >= 0 && x && y && pq && pulse_dtype_ok(dtype) && pulse_dtype_ok(pq_dtype), "xielu: bad arguments");
+    if (n == 0) return 0;
+    const int64_t blocks = (n + 255) / 256;
+    PULSE_REQUIRE(blocks < (1ll << 31), "xielu: too many elements");
+    PULSE_DISPATCH_DTYPE(dtype, T, PULSE_DISPATCH_DTYPE(pq_dtype, TP,
+        hipLaunchKernelGGL((xielu_kernel<T, TP>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
+                           static_cast<const T*>(x), static_cast<T*>(y), n, static_cast<const TP*>(pq))));
+    PULSE_LAUNCH_CHECK("xielu");
+    return 0;
+}

@@ -31,6 +31,8 @@ def expected_tensors(spec: ModelSpec) -> Dict[str, TensorSpec]:
         out[joined(spec.final_norm_prefix, name)] = ts
     for name, ts in HEADS.get(spec.head.kind).weight_specs(spec.head.params).items():
         out.setdefault(name, ts)
+    for name, rows in spec.offsets.items():
+        out[name] = TensorSpec((rows, spec.hidden_size), kind="linear", fan_in=4)
     return out
 
 
@@ -58,6 +60,7 @@ class CausalLM:
         self.blocks = [BLOCKS.get(layer.block.kind)(layer, build) for layer in spec.layers]
         self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm.params, spec.final_norm_prefix, build)
         self.head = HEADS.get(spec.head.kind)(spec.head.params, build, self.embedding)
+        self.offsets = {name: loader.get(name) for name in spec.offsets}
         self.vocab_size = spec.vocab_size
         self.hidden_size = spec.hidden_size
         self._clean: Optional[bool] = None
@@ -103,11 +106,16 @@ class CausalLM:
             # one gathers the wanted rows and stays a kernel of its own)
             follower = self.blocks[order[index + 1].layer] if index + 1 < len(order) else None
             stream.after_block = follower.entry_norm() if hasattr(follower, "entry_norm") else None
+            if run.offset is not None:
+                # (a sum: it may go in while an update is still pending; what was known about the rows no longer holds)
+                from ..ops import kernels
+                kernels.residual_add_row(stream.h, self.offsets[run.offset[0]][run.offset[1]])
+                stream.stats = stream.copy = None
             self.blocks[run.layer].forward(stream, ctx, cache_views[index])
         logits = torch.empty((ctx.num_wanted, self.vocab_size), dtype=torch.float32, device=self.device)
         if ctx.num_wanted == 0:
             return logits
         x = ws.buffer("model.final", ctx.num_wanted, self.hidden_size, self.act_dtype)
-        self.final_norm.apply(stream.h, stream.pending_for(self.final_norm), x, rows=ctx.want_rows)
+        stream.normed(self.final_norm, x, rows=ctx.want_rows)
         self.head.forward(x, logits)
         return logits

@@ -11,7 +11,7 @@ describes; configuration classes produce it, ``CausalLM`` consumes it.
 from __future__ import annotations
 
 from dataclasses import dataclass, field, replace
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, List, Optional, Tuple
 
 
 @dataclass(frozen=True)
@@ -61,10 +61,13 @@ class RunSpec:
 
     ``layer`` indexes ``ModelSpec.layers``.  ``cache_of`` is the index (in the
     order) of an earlier run whose cache this run reads instead of owning one.
+    ``offset`` = (tensor, row): that row of a tensor listed in ``ModelSpec.offsets`` is added to the residual of every
+    token right before the run (the marker of a pass over layers that run several times).
     """
 
     layer: int
     cache_of: Optional[int] = None
+    offset: Optional[Tuple[str, int]] = None
 
 
 @dataclass
@@ -84,6 +87,8 @@ class ModelSpec:
     # rows of the residual a token (hyper-connections keep several streams); the embedding fills them all, blocks and
     # the final norm must be of kinds that read that many
     streams: int = 1
+    # tensors [rows, hidden_size] whose rows runs add to the residual (``RunSpec.offset``): name -> rows
+    offsets: Dict[str, int] = field(default_factory=dict)
 
     def validate(self) -> None:
         if not self.layers:
@@ -93,6 +98,12 @@ class ModelSpec:
         for index, run in enumerate(self.order):
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"order[{index}] names layer {run.layer}, the model has {len(self.layers)}")
+            if run.offset is not None:
+                name, row = run.offset
+                if name not in self.offsets or not 0 <= row < self.offsets[name]:
+                    raise ValueError(f"order[{index}].offset names row {row} of '{name}', the model lists {self.offsets}")
+                if self.streams != 1:
+                    raise ValueError("offsets are added to a residual of one stream")
             if run.cache_of is not None:
                 if not 0 <= run.cache_of < index:
                     raise ValueError(f"order[{index}].cache_of must name an earlier run, got {run.cache_of}")

@@ -86,9 +86,9 @@ def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, bad_
 
 def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
                 out: torch.Tensor, rows: Optional[torch.Tensor] = None, write_back: bool = True,
-                weight_offset: float = 0.0) -> None:
-    """out[r] = rmsnorm(h[s] + delta[s]) * (weight_offset + weight), s = rows[r] or r; with write_back h[s] keeps the
-    sum.  ``weight_offset`` is 1 for a weight stored as its distance from one (added in float32), else 0.
+                weight_offset: float = 0.0, delta_scale: float = 1.0) -> None:
+    """out[r] = rmsnorm(h[s] + delta_scale * delta[s]) * (weight_offset + weight), s = rows[r] or r; with write_back
+    h[s] keeps the sum.  ``weight_offset`` is 1 for a weight stored as its distance from one (added in float32), else 0.
     ``delta`` may be float32 [parts, T, H]: the shares of a product whose inner dimension was split, added in order."""
     _gpu("add_rmsnorm", h, delta, weight, out, rows)
     _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "add_rmsnorm: h must be contiguous float32 [T, H]")
@@ -111,18 +111,27 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
     call("pulse_add_rmsnorm", _ptr(h), _ptr(delta), _i32(_tag(delta, "add_rmsnorm") if delta is not None else 0),
          _i32(parts), _i64(h.numel()), _ptr(rows), _ptr(weight), _i32(_tag(weight, "add_rmsnorm")), _ptr(out), _i32(_tag(out, "add_rmsnorm")),
          _i32(n_out), _i32(hidden), _f32(eps), _i32(1 if (write_back and delta is not None) else 0), _f32(weight_offset),
-         _stream())
+         _f32(delta_scale), _stream())
 
 
-def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
-    """h += delta; ``delta`` of the shape of h, or [parts, *h.shape] (added in order)."""
+def residual_add(h: torch.Tensor, delta: torch.Tensor, scale: float = 1.0) -> None:
+    """h += scale * delta; ``delta`` of the shape of h, or [parts, *h.shape] (added in order)."""
     _gpu("residual_add", h, delta)
     parts = delta.shape[0] if delta.dim() == h.dim() + 1 else 1
     _need(h.dtype == torch.float32 and h.is_contiguous() and delta.is_contiguous()
           and (delta.shape == h.shape or delta.shape[1:] == h.shape),
           "residual_add: h must be contiguous float32 and delta of the same shape (or several of them)")
     call("pulse_residual_add", _ptr(h), _ptr(delta), _i32(_tag(delta, "residual_add")), _i32(parts), _i64(h.numel()),
-         _stream())
+         _f32(scale), _stream())
+
+
+def residual_add_row(h: torch.Tensor, row: torch.Tensor) -> None:
+    """h[t] += row for every row t of h [T, H]; ``row`` holds H values."""
+    _gpu("residual_add_row", h, row)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous() and row.is_contiguous()
+          and row.numel() == h.shape[1], "residual_add_row: h must be contiguous float32 [T, H] and row hold H values")
+    call("pulse_residual_add_row", _ptr(h), _ptr(row), _i32(_tag(row, "residual_add_row")), _i64(h.numel()),
+         _i32(h.shape[1]), _stream())
 
 
 GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
@@ -474,8 +483,13 @@ def qk_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight: Optional[
 def attn_generic(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
                  vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
                  scale: float, window: int = 0, gate: Optional[torch.Tensor] = None, gate_width: int = 0,
-                 sink: Optional[torch.Tensor] = None, softcap: float = 0.0) -> None:
+                 sink: Optional[torch.Tensor] = None, softcap: float = 0.0, keep_first: int = 0,
+                 all_values: bool = False) -> None:
     """Paged causal attention, one wavefront per (token, head), float32 arithmetic.
+
+    ``keep_first`` > 0 (with a window): the request's first ``keep_first`` keys stay visible below the window.
+    ``all_values``: every query head's weights are applied to the values of all kv heads; ``out`` is then float32
+    [T, nq * nkv * d] (head h, value head c at (h * nkv + c) * d).  ``out`` may be float32 in any case.
 
     ``gate_width`` > 0: the gate holds a logit for each of the first ``gate_width`` channels of every head
     ([T, nq * gate_width]) instead of one a head.  ``sink`` float32 [nq]: exp(sink[h]) is one more term of head h's
@@ -486,9 +500,15 @@ def attn_generic(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, 
     """
     _gpu("attn_generic", q, out, kcache, vcache, positions, token_entry, block_table)
     tokens = q.shape[0]
-    _need(q.dim() == 2 and out.dim() == 2 and q.stride(1) == 1 and out.stride(1) == 1 and q.dtype == out.dtype,
-          "attn_generic: q and out must be matrices of one storage type with contiguous rows")
-    _need(q.shape[1] >= nq * d and out.shape[1] >= nq * d and out.shape[0] == tokens, "attn_generic: q/out too narrow")
+    out_f32 = out.dtype == torch.float32 and q.dtype != torch.float32
+    _need(q.dim() == 2 and out.dim() == 2 and q.stride(1) == 1 and out.stride(1) == 1
+          and (q.dtype == out.dtype or out_f32),
+          "attn_generic: q and out must be matrices with contiguous rows, out of q's storage type or float32")
+    _need(not all_values or (out.dtype == torch.float32 and gate is None),
+          "attn_generic: all values side by side come out in float32 and ungated")
+    out_width = nq * d * (nkv if all_values else 1)
+    _need(q.shape[1] >= nq * d and out.shape[1] >= out_width and out.shape[0] == tokens, "attn_generic: q/out too narrow")
+    _need(keep_first >= 0, "attn_generic: negative number of kept keys")
     pages, page_size = _check_cache("attn_generic", kcache, vcache, nkv, d)
     _int_vec("attn_generic: positions", positions, tokens)
     _int_vec("attn_generic: token_entry", token_entry, tokens)
@@ -505,11 +525,160 @@ def attn_generic(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, 
         _need(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == nq,
               f"attn_generic: the sinks must be float32 [{nq}]")
     gate_stride = 0 if gate is None else (gate.stride(0) if tokens > 1 else max(nq * max(1, gate_width), gate.shape[1]))
-    call("pulse_attn_generic", _ptr(q), _i64(q.stride(0)), _ptr(out), _i64(out.stride(0)), _i32(_tag(q, "attn_generic")),
+    o_stride = out.stride(0) if tokens > 1 else max(out_width, out.shape[1])
+    call("pulse_attn_generic_ex", _ptr(q), _i64(q.stride(0)), _ptr(out), _i64(o_stride), _i32(_tag(q, "attn_generic")),
          _ptr(kcache), _ptr(vcache), _i32(_tag(kcache, "attn_generic")), _ptr(positions), _ptr(token_entry),
          _ptr(block_table), _i32(block_table.shape[1]), _i32(tokens), _i32(nq), _i32(nkv), _i32(d), _i32(page_size),
          _i32(pages), _f32(scale), _i32(window), _ptr(gate), _i64(gate_stride),
-         _i32(gate_width if gate is not None else 0), _ptr(sink), _f32(softcap), _stream())
+         _i32(gate_width if gate is not None else 0), _ptr(sink), _f32(softcap), _i32(keep_first),
+         _i32(1 if all_values else 0), _i32(1 if out.dtype == torch.float32 else 0), _stream())
+
+
+def head_mix(x: torch.Tensor, mix: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, d: int, dv: int,
+             out_d: int, scale: float = 1.0) -> None:
+    """out[t, h, e] = scale * sum_g mix[h, g] * x[t, g, h // (heads // kv_heads), e] for e < dv, zero for dv <= e <
+    out_d: the heads' attention weights mixed behind the attention kernel (x float32 [T, heads * kv_heads * d], as
+    ``attn_generic`` leaves it with ``all_values``); out [T, heads * out_d], rows may be strided."""
+    _gpu("head_mix", x, mix, out)
+    tokens = x.shape[0]
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.shape[1] == heads * kv_heads * d,
+          f"head_mix: x must be contiguous float32 [{tokens}, {heads * kv_heads * d}]")
+    _need(mix.is_contiguous() and tuple(mix.shape) == (heads, heads), f"head_mix: mix must be [{heads}, {heads}]")
+    _need(out.dim() == 2 and out.shape[0] == tokens and out.shape[1] == heads * out_d and out.stride(1) == 1,
+          f"head_mix: out must be [{tokens}, {heads * out_d}] with contiguous rows")
+    stride = out.stride(0) if tokens > 1 else max(heads * out_d, out.shape[1])
+    call("pulse_head_mix", _ptr(x), _ptr(mix), _i32(_tag(mix, "head_mix")), _ptr(out), _i64(stride),
+         _i32(_tag(out, "head_mix")), _i32(tokens), _i32(heads), _i32(kv_heads), _i32(d), _i32(dv), _i32(out_d),
+         _f32(scale), _stream())
+
+
+def rotate_qk_rows(x: torch.Tensor, q0: int, k0: int, v0: int, out: torch.Tensor, heads: int, d: int, dv: int,
+                   cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rotary_dim: int, pairing: int,
+                   key_scale: float = 1.0) -> None:
+    """out [T, 2 heads d + heads dv] float32 = q, k, v of the projection output ``x`` (columns q0, k0, v0), the first
+    ``rotary_dim`` channels of every head of q and k turned by the tokens' tables, k times ``key_scale``."""
+    _gpu("rotate_qk_rows", x, out, cos, sin)
+    tokens = x.shape[0]
+    rot = rotary_dim if cos is not None else 0
+    _need(x.dim() == 2 and x.stride(1) == 1, "rotate_qk_rows: x must have contiguous rows")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (tokens, 2 * heads * d + heads * dv),
+          f"rotate_qk_rows: out must be contiguous float32 [{tokens}, {2 * heads * d + heads * dv}]")
+    if rot:
+        for t in (cos, sin):
+            _need(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (tokens, rot // 2),
+                  f"rotate_qk_rows: the tables must be contiguous float32 [{tokens}, {rot // 2}]")
+    stride = x.stride(0) if tokens > 1 else x.shape[1]
+    call("pulse_rotate_qk_rows", _ptr(x), _i64(stride), _i32(_tag(x, "rotate_qk_rows")), _i32(q0), _i32(k0), _i32(v0),
+         _ptr(out), _i32(tokens), _i32(heads), _i32(d), _i32(dv), _ptr(cos if rot else None), _ptr(sin if rot else None),
+         _i32(rot), _i32(pairing), _f32(key_scale), _stream())
+
+
+GATE_FORMS = {"sigmoid": 0, "silu": 1}
+
+
+def group_norm_gate(o: torch.Tensor, weight: Optional[torch.Tensor], gate: Optional[torch.Tensor], out: torch.Tensor,
+                    groups: int, eps: float, scale: float = 1.0, gate_form: str = "sigmoid") -> None:
+    """Every one of the ``groups`` equal parts of a row of ``o`` (float32) divided by its own root mean square, times
+    ``weight`` (optional, one a column), times sigmoid(gate) or silu(gate) (optional), times ``scale``; one rounding."""
+    _gpu("group_norm_gate", o, weight, gate, out)
+    tokens, width = o.shape
+    _need(groups > 0 and width % groups == 0, f"group_norm_gate: {width} columns in {groups} groups")
+    _need(gate_form in GATE_FORMS, f"group_norm_gate: a gate is one of {sorted(GATE_FORMS)}, not '{gate_form}'")
+    _need(o.dtype == torch.float32 and o.stride(1) == 1, "group_norm_gate: o must be float32 with contiguous rows")
+    _need(out.dim() == 2 and out.shape[0] == tokens and out.shape[1] == width and out.stride(1) == 1,
+          f"group_norm_gate: out must be [{tokens}, {width}] with contiguous rows")
+    _need(gate is None or (gate.shape == out.shape and gate.stride(1) == 1 and gate.dtype == out.dtype),
+          "group_norm_gate: the gate must have out's shape and storage type")
+    _need(weight is None or (weight.numel() == width and weight.is_contiguous()),
+          f"group_norm_gate: weight must hold {width} values")
+    row = lambda t: t.stride(0) if tokens > 1 else max(width, t.shape[1])
+    call("pulse_group_norm_gate", _ptr(o), _i64(row(o)), _ptr(weight),
+         _i32(_tag(weight, "group_norm_gate") if weight is not None else 0), _ptr(gate),
+         _i64(row(gate) if gate is not None else 0), _ptr(out), _i64(row(out)), _i32(_tag(out, "group_norm_gate")),
+         _i32(tokens), _i32(groups), _i32(width // groups), _f32(eps), _f32(scale), _i32(GATE_FORMS[gate_form]), _stream())
+
+
+def latent_rows(x: torch.Tensor, q0: int, c0: int, q: torch.Tensor, norm_weight: torch.Tensor, cos: torch.Tensor,
+                sin: torch.Tensor, pairing: int, kcache: torch.Tensor, vcache: torch.Tensor, positions: torch.Tensor,
+                token_entry: torch.Tensor, block_table: torch.Tensor, heads: int, d: int, rot: int, rank: int,
+                stored: int, eps: float, write: bool = True) -> None:
+    """Latent attention's preparation: the normed latent row and the turned key part of every token into the pages
+    (keys [pages, 1, page, stored] = [c | turned | 0], values [pages, 1, stored, page] = [c | 0]) and the queries'
+    turned parts into ``q`` [T, heads * stored] at rank .. rank + rot of every head (zeros behind)."""
+    _gpu("latent_rows", x, q, norm_weight, cos, sin, kcache, vcache, positions, token_entry, block_table)
+    tokens = x.shape[0]
+    _need(x.dim() == 2 and x.stride(1) == 1 and q.dim() == 2 and q.stride(1) == 1 and q.dtype == x.dtype
+          and q.shape[0] == tokens and q.shape[1] >= heads * stored, "latent_rows: x and q must be matrices of one type")
+    pages, page_size = _check_cache("latent_rows", kcache, vcache, 1, stored)
+    _int_vec("latent_rows: positions", positions, tokens)
+    _int_vec("latent_rows: token_entry", token_entry, tokens)
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+          "latent_rows: block_table must be contiguous int32 [entries, width]")
+    _need(norm_weight.numel() == rank and norm_weight.is_contiguous(), f"latent_rows: the norm's weight must hold {rank} values")
+    for t in (cos, sin):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (tokens, rot // 2),
+              f"latent_rows: the tables must be contiguous float32 [{tokens}, {rot // 2}]")
+    call("pulse_latent_rows", _ptr(x), _i64(x.stride(0) if tokens > 1 else x.shape[1]), _i32(_tag(x, "latent_rows")),
+         _i32(q0), _i32(c0), _ptr(q), _i64(q.stride(0) if tokens > 1 else q.shape[1]), _ptr(norm_weight),
+         _i32(_tag(norm_weight, "latent_rows")), _ptr(cos), _ptr(sin), _i32(pairing), _ptr(kcache), _ptr(vcache),
+         _i32(_tag(kcache, "latent_rows")), _ptr(positions), _ptr(token_entry), _ptr(block_table),
+         _i32(block_table.shape[1]), _i32(tokens), _i32(heads), _i32(d), _i32(rot), _i32(rank), _i32(stored),
+         _i32(page_size), _i32(pages), _f32(eps), _i32(1 if write else 0), _stream())
+
+
+def latent_absorb(x: torch.Tensor, q0: int, q_head: int, w_uk: torch.Tensor, q: torch.Tensor, stored: int, heads: int,
+                  d: int, rank: int) -> None:
+    """q[t, h * stored + r] = sum_e x[t, q0 + h * q_head + e] * w_uk[h * d + e, r]: a head's plain query part taken
+    into the latent space (float32 sums, one rounding)."""
+    _gpu("latent_absorb", x, w_uk, q)
+    tokens = x.shape[0]
+    _need(x.dim() == 2 and x.stride(1) == 1 and q.dim() == 2 and q.stride(1) == 1 and q.dtype == x.dtype
+          and q.shape[0] == tokens and q.shape[1] >= heads * stored, "latent_absorb: x and q must be matrices of one type")
+    _need(w_uk.is_contiguous() and tuple(w_uk.shape) == (heads * d, rank), f"latent_absorb: w_uk must be [{heads * d}, {rank}]")
+    call("pulse_latent_absorb", _ptr(x), _i64(x.stride(0) if tokens > 1 else x.shape[1]), _i32(_tag(x, "latent_absorb")),
+         _i32(q0), _i32(q_head), _ptr(w_uk), _i32(_tag(w_uk, "latent_absorb")), _ptr(q),
+         _i64(q.stride(0) if tokens > 1 else q.shape[1]), _i32(stored), _i32(tokens), _i32(heads), _i32(d), _i32(rank),
+         _stream())
+
+
+def latent_expand(o: torch.Tensor, stored: int, w_uv: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor,
+                  heads: int, dv: int, rank: int, scale: float = 1.0) -> None:
+    """out[t, h * dv + e] = scale * (sum_r w_uv[h * dv + e, r] * o[t, h * stored + r]) * sigmoid(gate[t, h * dv + e]):
+    the heads' weighted latent rows expanded to their values, gated channel by channel; one rounding."""
+    _gpu("latent_expand", o, w_uv, gate, out)
+    tokens = o.shape[0]
+    _need(o.dim() == 2 and o.stride(1) == 1 and o.shape[1] >= heads * stored, "latent_expand: o too narrow")
+    _need(w_uv.is_contiguous() and tuple(w_uv.shape) == (heads * dv, rank), f"latent_expand: w_uv must be [{heads * dv}, {rank}]")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == tokens and out.shape[1] >= heads * dv,
+          "latent_expand: out too narrow")
+    _need(gate is None or (gate.dtype == out.dtype and gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[0] == tokens
+                           and gate.shape[1] >= heads * dv), "latent_expand: the gate must be of out's type and width")
+    row = lambda t: t.stride(0) if tokens > 1 else t.shape[1]
+    call("pulse_latent_expand", _ptr(o), _i64(row(o)), _i32(_tag(o, "latent_expand")), _i32(stored), _ptr(w_uv),
+         _i32(_tag(w_uv, "latent_expand")), _ptr(gate), _i64(row(gate) if gate is not None else 0), _ptr(out),
+         _i64(row(out)), _i32(_tag(out, "latent_expand")), _i32(tokens), _i32(heads), _i32(dv), _i32(rank), _f32(scale),
+         _stream())
+
+
+def xielu(x: torch.Tensor, out: torch.Tensor, pq: torch.Tensor) -> None:
+    """out = a z^2 + z / 2 for z > 0, else b (exp(z) - 1 - z) + z / 2, a = softplus(pq[0]), b = 1/2 + softplus(pq[1])."""
+    _gpu("xielu", x, out, pq)
+    _need(x.shape == out.shape and x.dtype == out.dtype and x.is_contiguous() and out.is_contiguous(),
+          "xielu: x and out must be contiguous and alike")
+    _need(pq.numel() == 2 and pq.is_contiguous(), "xielu: the activation has two numbers")
+    call("pulse_xielu", _ptr(x), _ptr(out), _i32(_tag(x, "xielu")), _i64(x.numel()), _ptr(pq), _i32(_tag(pq, "xielu")),
+         _stream())
+
+
+def token_gate_add(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, acc: torch.Tensor) -> None:
+    """acc[t] += sigmoid(w . x[t]) * y[t]; acc float32 [T, H], x and y [T, H] of one storage type, w holds H values."""
+    _gpu("token_gate_add", x, w, y, acc)
+    tokens, hidden = x.shape
+    _need(x.is_contiguous() and y.is_contiguous() and acc.is_contiguous() and y.shape == x.shape and y.dtype == x.dtype
+          and acc.shape == x.shape and acc.dtype == torch.float32, "token_gate_add: x, y [T, H] alike, acc float32 [T, H]")
+    _need(w.numel() == hidden and w.is_contiguous(), f"token_gate_add: w must hold {hidden} values")
+    call("pulse_token_gate_add", _ptr(x), _ptr(w), _i32(_tag(w, "token_gate_add")), _ptr(y), _i32(_tag(x, "token_gate_add")),
+         _ptr(acc), _i32(tokens), _i32(hidden), _stream())
 
 
 def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.Tensor] = None,

@@ -1,6 +1,6 @@
 from .base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, BuildContext, EntryMeta,
                    PagedCacheView, Part, Registry, ResidualStream, StateView, StepContext, Workspace)
-from . import attention, attention_rows, block, embedding, lightning, mamba, mlp, moe, norm, rope, side_by_side  # noqa: F401  (registers the built-in parts)
+from . import attention, attention_rows, block, embedding, latent, lightning, mamba, mlp, moe, norm, rope, side_by_side  # noqa: F401  (registers the built-in parts)
 
 __all__ = ["BLOCKS", "EMBEDDINGS", "FEED_FORWARDS", "HEADS", "MIXERS", "NORMS", "POSITIONS", "BuildContext", "EntryMeta",
            "PagedCacheView", "Part", "Registry", "ResidualStream", "StateView", "StepContext", "Workspace"]

@@ -10,7 +10,11 @@ mean square, no weights; the same before or after the rotation, which keeps a he
 float32 before their one rounding); ``output_gate``: "channel": the heads' outputs are multiplied element by element
 by sigmoid(Wg x), Wg [heads * value_dim, hidden] (tensor ``gate``), whose rows ride behind q, k and v in the stacked
 projection and whose sigmoid the attention kernels apply as they store; ``score_cap`` and ``sink`` as for
-``attention``.
+``attention``; ``keep_first`` (with a window): a request's first ``keep_first`` tokens stay visible below the window,
+at their true positions; ``talk``: the heads' attention weights are mixed before they meet the values, weight_h <-
+sum_g T[h, g] weight_g with T the tensor ``talk`` [heads, heads] (a sink's share is not mixed); head h applies its
+mixed weights to the values of its own kv head.  Both run on the generic attention kernel: with ``talk`` it leaves
+every head's weights applied to the values of every kv head, in float32, and ``pulse_head_mix`` forms the sums.
 
 Keys and values are stored with one width D = max(head_dim, value_dim) rounded up to a multiple of 16, the missing
 channels as zeros: zero key channels add nothing to a score, and zero value channels come out as zeros, which meet
@@ -39,7 +43,7 @@ def stored_width(d: int, dv: int) -> int:
 @MIXERS.register("attention_rows")
 class RowPreparedAttention(PagedAttention):
     NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "q_bias": "q.b", "k_bias": "k.b", "v_bias": "v.b",
-             "q_norm": "q.norm", "k_norm": "k.norm", "gate": "g", "sink": "sink"}
+             "q_norm": "q.norm", "k_norm": "k.norm", "gate": "g", "sink": "sink", "talk": "talk"}
 
     @classmethod
     def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
@@ -63,6 +67,8 @@ class RowPreparedAttention(PagedAttention):
             specs[n["gate"]] = TensorSpec((nq * dv, hidden), fan_in=hidden)
         if params.get("sink", False):
             specs[n["sink"]] = TensorSpec((nq,), kind="linear", fan_in=4)
+        if params.get("talk", False):
+            specs[n["talk"]] = TensorSpec((nq, nq), kind="linear", fan_in=nq)
         return specs
 
     @classmethod
@@ -72,13 +78,15 @@ class RowPreparedAttention(PagedAttention):
         cost = Part.step_cost.__func__(cls, params, entries, weight_bytes, cache_bytes)
         nq, nkv, d, window = params["num_heads"], params["num_kv_heads"], params["head_dim"], params.get("window")
         dv = params.get("value_dim", d)
+        first = int(params.get("keep_first", 0) or 0) if window else 0
+        fan = nkv if params.get("talk", False) else 1     # every head's weights meet the values of every kv head
         for start, count in entries:
             seen = 0
             for p in range(start, start + count):
-                seen += min(p + 1, window) if window else p + 1
-            cost.flops += 2.0 * nq * (d + dv) * seen
+                seen += min(p + 1, window + first) if window else p + 1
+            cost.flops += 2.0 * nq * (d + dv * fan) * seen
             context = start + count
-            kept = min(context, window + count - 1) if window else context
+            kept = min(context, window + first + count - 1) if window else context
             cost.cache_bytes += 2.0 * nkv * stored_width(d, dv) * cache_bytes * kept
         return cost
 
@@ -104,6 +112,14 @@ class RowPreparedAttention(PagedAttention):
         if gate not in (False, None, "channel"):
             raise ValueError(f"attention_rows has an output gate by 'channel' or none, got {gate!r}")
         self.channel_gate = gate == "channel"
+        self.keep_first = int(params.get("keep_first", 0) or 0)
+        if self.keep_first < 0:
+            raise ValueError(f"the number of kept first tokens must not be negative, got {self.keep_first}")
+        if self.window is None:
+            self.keep_first = 0
+        self.talks = bool(params.get("talk", False))
+        if self.talks and self.channel_gate:
+            raise ValueError("attention_rows has no kernel for mixed heads with an output gate")
         self._read_score_form(params)
         self.eps = float(params.get("qk_norm_eps", 0.0))
         self.out_scale = float(params.get("out_scale", 1.0))
@@ -119,6 +135,7 @@ class RowPreparedAttention(PagedAttention):
         self.kv_cols = self.nq * self.qk_dim + self.nkv * (self.qk_dim + self.v_dim)   # where the gate's columns start
         self.gate_width = self.v_dim if self.channel_gate else 0
         self.sink = self._load_sink(load, n["sink"]) if params.get("sink", False) else None
+        self.talk = load.get(n["talk"]) if self.talks else None
         self.biases = tuple(load.get(n[k]) for k in ("q_bias", "k_bias", "v_bias")) if params.get("bias", False) else None
         self.norm_weights = (load.get(n["q_norm"]), load.get(n["k_norm"])) if self.row_norm else None
         o = load.get(n["o"])
@@ -142,7 +159,11 @@ class RowPreparedAttention(PagedAttention):
     records_cleanly = True
 
     def cache_spec(self) -> PagedKVSpec:
-        return PagedKVSpec(self.nkv, self.d, int(self.window) if self.window is not None else None)
+        return PagedKVSpec(self.nkv, self.d, int(self.window) if self.window is not None else None, self.keep_first)
+
+    def uses_matrix_cores(self, q: torch.Tensor, cache: PagedCacheView) -> bool:
+        # (kept first tokens and mixed heads are the generic kernel's)
+        return not (self.keep_first or self.talks) and super().uses_matrix_cores(q, cache)
 
     def out_weight(self) -> torch.Tensor:
         return self._o_weight
@@ -165,7 +186,22 @@ class RowPreparedAttention(PagedAttention):
                          ctx.token_entry, table, write_kv=write, value_scale=self.out_scale,
                          norm="head" if self.head_norm else self.row_norm)
         gate = qkv[:, self.kv_cols:self.kv_cols + self.nq * self.v_dim] if self.channel_gate else None
-        self.attend(q, out, ctx, cache, table, gate=gate)
+        if not (self.keep_first or self.talks):
+            self.attend(q, out, ctx, cache, table, gate=gate)
+            return
+        window = int(self.window) if self.window is not None else 0
+        if not self.talks:
+            kernels.attn_generic(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
+                                 ctx.token_entry, table, self.scale, window, gate=gate, gate_width=self.gate_width,
+                                 sink=self.sink, softcap=self.score_cap, keep_first=self.keep_first)
+            return
+        # every head's weights on every kv head's values, then the sums over heads that the mixing matrix asks for
+        # (the branch's factor is already in the stored values)
+        each = ws.buffer("attention_rows.each", tokens, self.nq * self.nkv * self.d, torch.float32)
+        kernels.attn_generic(q, each, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
+                             ctx.token_entry, table, self.scale, window, sink=self.sink, softcap=self.score_cap,
+                             keep_first=self.keep_first, all_values=True)
+        kernels.head_mix(each, self.talk, out, self.nq, self.nkv, self.d, self.v_dim, self.d)
 
     def decodes_from_raw(self, ctx, cache, qkv, tables) -> bool:
         return False

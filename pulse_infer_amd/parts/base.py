@@ -244,6 +244,7 @@ class ResidualStream:
     def __init__(self, h: torch.Tensor):
         self.h = h
         self.pending: Optional[torch.Tensor] = None
+        self.pending_scale: float = 1.0   # the factor with which ``pending`` enters the sum (a block's multiplier)
         self.stats: Optional[RowStats] = None
         self.after_block: Any = None   # the norm that reads the residual first once the block in hand is through
                                        # (set by whoever runs the blocks; None: unknown, or no norm)
@@ -254,8 +255,13 @@ class ResidualStream:
         """The update not yet added, in a form ``norm`` takes: an update in parts ([parts, T, H] float32, the shares of
         a product whose inner dimension was split) is added to ``h`` first unless the norm says ``takes_parts``."""
         pending, self.pending = self.pending, None
+        scale, self.pending_scale = self.pending_scale, 1.0
         if pending is not None:
             self.copy = None
+        if pending is not None and scale != 1.0:   # (only ``normed`` hands a factor on to a norm that takes one)
+            from ..ops import kernels
+            kernels.residual_add(self.h, pending, scale)
+            return None
         if isinstance(pending, StreamUpdate):
             if getattr(norm, "takes_streams", False):
                 return pending
@@ -267,8 +273,16 @@ class ResidualStream:
             return None
         return pending
 
-    def normed(self, norm: Any, out: torch.Tensor) -> torch.Tensor:
-        norm.apply(self.h, self.pending_for(norm), out)
+    def normed(self, norm: Any, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """out = norm(h + what is pending), of all rows or of the gathered ``rows``."""
+        extra = {} if rows is None else {"rows": rows}
+        if (self.pending is not None and self.pending_scale != 1.0 and getattr(norm, "takes_scale", False)
+                and isinstance(self.pending, torch.Tensor)):
+            pending, scale = self.pending, self.pending_scale
+            self.pending, self.pending_scale, self.copy = None, 1.0, None
+            norm.apply(self.h, pending, out, delta_scale=scale, **extra)
+            return out
+        norm.apply(self.h, self.pending_for(norm), out, **extra)
         return out
 
     def lazy(self, norm: Any) -> Optional[LazyNorm]:
@@ -286,13 +300,14 @@ class ResidualStream:
             if isinstance(self.pending, StreamUpdate):
                 self.pending.apply_to(self.h)
             else:
-                kernels.residual_add(self.h, self.pending)
+                kernels.residual_add(self.h, self.pending, self.pending_scale)
             self.pending = None
+            self.pending_scale = 1.0
             self.copy = None
 
-    def push(self, delta: Any) -> None:
+    def push(self, delta: Any, scale: float = 1.0) -> None:
         """Hand over an update ([T, H], or [parts, T, H] float32 to be added in order); None or RowStats mean the part
-        has already added it to ``h``."""
+        has already added it to ``h``.  ``scale``: the update enters the sum times this factor."""
         self.copy = None
         if isinstance(delta, RowStats):
             self.stats = delta
@@ -305,8 +320,9 @@ class ResidualStream:
             if isinstance(self.pending, StreamUpdate):
                 self.pending.apply_to(self.h)
             else:
-                kernels.residual_add(self.h, self.pending)
+                kernels.residual_add(self.h, self.pending, self.pending_scale)
         self.pending = delta
+        self.pending_scale = float(scale)
 
 
 @dataclass

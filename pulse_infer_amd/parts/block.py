@@ -4,6 +4,9 @@
 (reference: src/model/qwen3/model.cpp:779-923).  The additions are deferred into
 the next norm's kernel through ``ResidualStream``.
 
+``prenorm_scaled``: h <- h + m mixer(norm_a(h)); h <- h + m ffn(norm_b(h)) with one multiplier m on both
+updates; the feed-forward may be absent.
+
 ``parallel``: n = norm(h); h <- h + (mixer(n) + ffn(n)): one norm, whose output both
 sublayers read; a layer may have no feed-forward (``LayerSpec.ffn`` None), then
 h <- h + mixer(norm(h)).
@@ -108,6 +111,63 @@ class PreNormBlock(Part):
             stream.push(self.ffn.forward(x, ctx, residual=stream.h, **self._told(stream.after_block)))
         else:
             stream.push(self.ffn.forward(x, ctx))
+
+
+@BLOCKS.register("prenorm_scaled")
+class ScaledPreNormBlock(PreNormBlock):
+    """The pre-norm arrangement with a multiplier on the sublayers' results: h <- h + m * mixer(norm_a(h)), then
+    h <- h + m * ffn(norm_b(h)).  Block parameters: ``mixer_norm`` / ``ffn_norm`` (the norms' tensor prefixes below the
+    layer's) and ``residual_scale`` = m (default 1).  A layer without a feed-forward ends after the mixer.
+
+    The multiplied update is added inside the kernel of the norm that reads the residual next (a norm that says
+    ``takes_scale``), in float32; weights stay what the checkpoint holds.  A feed-forward may hand back two updates."""
+
+    @classmethod
+    def layer_weight_specs(cls, layer: LayerSpec) -> Dict[str, TensorSpec]:
+        p = layer.block.params
+        out: Dict[str, TensorSpec] = {}
+        places = ["mixer_norm"] + (["ffn_norm"] if layer.ffn is not None else [])
+        for which in places:
+            norm = layer.norm(which)
+            for name, spec in NORMS.get(norm.kind).weight_specs(norm.params).items():
+                out[joined(joined(layer.prefix, p[which]), name)] = spec
+        parts = [(layer.mixer, MIXERS)] + ([(layer.ffn, FEED_FORWARDS)] if layer.ffn is not None else [])
+        for part, registry in parts:
+            sub = joined(layer.prefix, part.params.get("prefix", ""))
+            for name, spec in registry.get(part.kind).weight_specs(part.params).items():
+                out[joined(sub, name)] = spec
+        return out
+
+    def __init__(self, layer: LayerSpec, build: BuildContext):
+        p = layer.block.params
+        self.residual_scale = float(p.get("residual_scale", 1.0))
+        norm = layer.norm("mixer_norm")
+        self.mixer_norm = NORMS.get(norm.kind)(norm.params, joined(layer.prefix, p["mixer_norm"]), build)
+        self.mixer = MIXERS.get(layer.mixer.kind)(layer.mixer.params,
+                                                  joined(layer.prefix, layer.mixer.params.get("prefix", "")), build)
+        self.ffn = self.ffn_norm = None
+        if layer.ffn is not None:
+            norm = layer.norm("ffn_norm")
+            self.ffn_norm = NORMS.get(norm.kind)(norm.params, joined(layer.prefix, p["ffn_norm"]), build)
+            self.ffn = FEED_FORWARDS.get(layer.ffn.kind)(layer.ffn.params,
+                                                         joined(layer.prefix, layer.ffn.params.get("prefix", "")), build)
+        self.act_dtype = build.act_dtype
+
+    def records_cleanly(self) -> bool:
+        return all(says(part, "records_cleanly")
+                   for part in (self.mixer, self.ffn, self.mixer_norm, self.ffn_norm) if part is not None)
+
+    def _push(self, stream: ResidualStream, update: Any) -> None:
+        first, second = update if isinstance(update, tuple) else (update, None)
+        stream.push(first, self.residual_scale)
+        if second is not None:
+            stream.push(second, self.residual_scale)
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Any) -> None:
+        x = ctx.workspace.buffer("block.normed", ctx.num_tokens, stream.h.shape[1], self.act_dtype)
+        self._push(stream, self.mixer.forward(stream.normed(self.mixer_norm, x), ctx, cache))
+        if self.ffn is not None:
+            self._push(stream, self.ffn.forward(stream.normed(self.ffn_norm, x), ctx))
 
 
 @BLOCKS.register("parallel")

@@ -13,6 +13,14 @@ the one rounding are a second kernel.
 Parameters: ``hidden_size``, ``num_heads``, ``head_dim``, ``value_dim``, ``decay`` (one number a head), ``norm_eps``,
 ``activation`` ("silu" or "none"), ``names`` (tensor names below the prefix), ``out_scale`` (a factor on the result).
 
+Variations ("retention" is the combination of all of them): ``position``: a position encoding of the model whose
+rotation turns the first channels of every head of q and k (activation "none" only); ``key_scale``: a factor on k,
+after the rotation; ``norm``: "all" (default: the heads of a token normed together) or "head" (every head divided by
+its own root mean square); ``norm_weight`` (default True; False: the norm has no weight and no tensor);
+``gate_activation``: "sigmoid" (default) or "silu".  With a rotation or a key factor q, k and v go from the
+projection's output into float32 rows first (``pulse_rotate_qk_rows``), which the walk reads: nothing behind the
+projection is rounded before it enters the recurrence.
+
 The part keeps a ``StateSpec`` per run.  It also answers the protocol of a branch of ``side_by_side``:
 ``inner_width``, ``out_weight()`` and ``forward_inner(x, ctx, cache, out)``.
 """
@@ -41,14 +49,16 @@ class LightningAttention(Part):
     def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
         hidden, heads, d, dv = (params[k] for k in ("hidden_size", "num_heads", "head_dim", "value_dim"))
         n = cls.tensor_names(params)
-        return {
+        specs = {
             n["q"]: TensorSpec((heads * d, hidden), fan_in=hidden),
             n["k"]: TensorSpec((heads * d, hidden), fan_in=hidden),
             n["v"]: TensorSpec((heads * dv, hidden), fan_in=hidden),
             n["gate"]: TensorSpec((heads * dv, hidden), fan_in=hidden),
             n["o"]: TensorSpec((hidden, heads * dv), fan_in=heads * dv),
-            n["norm"]: TensorSpec((heads * dv,), kind="norm"),
         }
+        if params.get("norm_weight", True):
+            specs[n["norm"]] = TensorSpec((heads * dv,), kind="norm")
+        return specs
 
     @classmethod
     def step_cost(cls, params: Dict[str, Any], entries: List[Tuple[int, int]], weight_bytes: int,
@@ -77,12 +87,26 @@ class LightningAttention(Part):
             raise ValueError(f"lightning attention has no kernel for activation '{self.activation}'")
         self.eps = float(params["norm_eps"])
         self.out_scale = float(params.get("out_scale", 1.0))
+        self.position = params.get("position")
+        self.encodings = build.positions
+        if self.position is not None and self.position not in self.encodings:
+            raise KeyError(f"lightning attention refers to position encoding '{self.position}', the model defines "
+                           f"{sorted(self.encodings)}")
+        if self.position is not None and self.activation != "none":
+            raise ValueError("lightning attention turns q and k only as they are projected (activation 'none')")
+        self.key_scale = float(params.get("key_scale", 1.0))
+        self.norm_over = params.get("norm", "all")
+        if self.norm_over not in ("all", "head"):
+            raise ValueError(f"lightning attention norms 'all' heads together or every 'head', not '{self.norm_over}'")
+        self.gate_activation = params.get("gate_activation", "sigmoid")
+        if self.gate_activation not in kernels.GATE_FORMS:
+            raise ValueError(f"a gate is one of {sorted(kernels.GATE_FORMS)}, not '{self.gate_activation}'")
         self.decay = torch.tensor(decay, dtype=torch.float32, device=build.device)
         load = build.loader
         self.names = {k: joined(prefix, v) for k, v in self.tensor_names(params).items()}
         n = self.names
         self.proj = Linear(load.get_concat([n["q"], n["k"], n["v"], n["gate"]]), build.mode)
-        self.norm_weight = load.get(n["norm"])
+        self.norm_weight = load.get(n["norm"]) if params.get("norm_weight", True) else None
         self._o_weight = load.get(n["o"])
         self._o = None
         self.mode = build.mode
@@ -120,9 +144,22 @@ class LightningAttention(Part):
             walkers = pieces.numel() // 4
             scratch = ws.buffer("lightning.pieces", walkers, self.heads * self.d * self.dv, torch.float32)
         groups = kernels.lightning_row_groups(walkers, self.heads, self.d, self.dv)
-        kernels.lightning_scan(y, 0, hd, 2 * hd, o, cache.state, self.decay, ctx.entry_first_row, ctx.entry_start,
+        rows = y
+        if self.position is not None or self.key_scale != 1.0:
+            tables = ctx.position_product(self.position, self.encodings) if self.position is not None else None
+            rows = ws.buffer("lightning.rows", tokens, 2 * hd + hv, torch.float32)
+            kernels.rotate_qk_rows(y, 0, hd, 2 * hd, rows, self.heads, self.d, self.dv,
+                                   tables.cos if tables is not None else None, tables.sin if tables is not None else None,
+                                   tables.rotary_dim if tables is not None else 0,
+                                   tables.pairing if tables is not None else 0, self.key_scale)
+        kernels.lightning_scan(rows, 0, hd, 2 * hd, o, cache.state, self.decay, ctx.entry_first_row, ctx.entry_start,
                                ctx.entry_slot, self.heads, self.d, self.dv, self.activation, groups, pieces, scratch)
-        kernels.gated_rmsnorm(o, self.norm_weight, y[:, 2 * hd + hv:], out, self.eps, self.out_scale)
+        gate = y[:, 2 * hd + hv:]
+        if self.norm_over == "all" and self.norm_weight is not None and self.gate_activation == "sigmoid":
+            kernels.gated_rmsnorm(o, self.norm_weight, gate, out, self.eps, self.out_scale)
+        else:
+            kernels.group_norm_gate(o, self.norm_weight, gate, out, self.heads if self.norm_over == "head" else 1,
+                                    self.eps, self.out_scale, self.gate_activation)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: StateView) -> torch.Tensor:
         if self._o is None:

@@ -98,9 +98,12 @@ class GatedMLP(Part):
 @FEED_FORWARDS.register("mlp")
 class PlainMLP(Part):
     """down(act(up(x))), no gate and no biases.  Parameters: ``hidden_size``, ``intermediate_size``, ``activation``
-    ("relu2": the square of relu, "gelu_tanh", "silu"), ``names`` (``up``, ``down``)."""
+    ("relu2": the square of relu, "gelu_tanh", "silu", "xielu": a z^2 + z / 2 for z > 0 and b (exp(z) - 1 - z) + z / 2
+    below, a = softplus(p), b = 1/2 + softplus(q) with the two learned numbers p, q in the tensor ``act``), ``names``
+    (``up``, ``down``, ``act``)."""
 
-    NAMES = {"up": "up", "down": "down"}
+    NAMES = {"up": "up", "down": "down", "act": "act"}
+    LEARNED = ("xielu",)    # activations with numbers of their own
 
     @classmethod
     def tensor_names(cls, params: Dict[str, Any]) -> Dict[str, str]:
@@ -110,16 +113,21 @@ class PlainMLP(Part):
     def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
         hidden, inter = params["hidden_size"], params["intermediate_size"]
         names = cls.tensor_names(params)
-        return {names["up"]: TensorSpec((inter, hidden), fan_in=hidden),
-                names["down"]: TensorSpec((hidden, inter), fan_in=inter)}
+        specs = {names["up"]: TensorSpec((inter, hidden), fan_in=hidden),
+                 names["down"]: TensorSpec((hidden, inter), fan_in=inter)}
+        if params.get("activation", "relu2") in cls.LEARNED:
+            specs[names["act"]] = TensorSpec((2,), kind="linear", fan_in=4)
+        return specs
 
     def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
         self.hidden = int(params["hidden_size"])
         self.inter = int(params["intermediate_size"])
         self.activation = params.get("activation", "relu2")
-        if self.activation not in kernels.ACTIVATIONS:
-            raise ValueError(f"mlp has no kernel for activation '{self.activation}' (known: {sorted(kernels.ACTIVATIONS)})")
+        if self.activation not in kernels.ACTIVATIONS and self.activation not in self.LEARNED:
+            raise ValueError(f"mlp has no kernel for activation '{self.activation}' "
+                             f"(known: {sorted(list(kernels.ACTIVATIONS) + list(self.LEARNED))})")
         names = {k: joined(prefix, v) for k, v in self.tensor_names(params).items()}
+        self.act_numbers = build.loader.get(names["act"]) if self.activation in self.LEARNED else None
         self.up = Linear(build.loader.get(names["up"]), build.mode)
         self.down = Linear(build.loader.get(names["down"]), build.mode)
         self.act_dtype = build.act_dtype
@@ -131,5 +139,8 @@ class PlainMLP(Part):
         ws = ctx.workspace
         z = ws.buffer("mlp.act", tokens, self.inter, self.act_dtype)
         self.up.forward(x, z)
-        kernels.activation(z, z, self.activation)
+        if self.act_numbers is not None:
+            kernels.xielu(z, z, self.act_numbers)
+        else:
+            kernels.activation(z, z, self.activation)
         return self.down.forward(z, ws.buffer("mlp.out", tokens, self.hidden, self.act_dtype))

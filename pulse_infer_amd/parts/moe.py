@@ -14,7 +14,9 @@ correction tensor exists), ``shared_size`` (None: no shared expert), ``names``: 
 (default True; False: the weights are the chosen scores as they are); ``weight_on``: "output" (default) or "input" (an
 expert is fed weight * x, and the experts' results are added as they are); ``expert_activation``: "silu" (default) or
 "clamped_swish" with ``limit``: g = min(gate x, limit), u = clamp(up x, -limit, limit), down(g * sigmoid(1.702 g) *
-(u + 1)).
+(u + 1)); ``shared_gate`` (default False): the shared expert's result is multiplied by sigmoid(w_sg . x), one number a
+token, with w_sg the tensor ``shared_gate`` [1, hidden] below the shared expert's prefix (the product then goes into
+the routed float32 sum and the part hands back one update).
 
 The experts' weights are stacked at load time ([experts, rows, columns]).  ``forward`` returns the routed part
 (float32) and the shared expert's part as two updates that the block adds.
@@ -34,7 +36,7 @@ from .mlp import GatedMLP
 @FEED_FORWARDS.register("routed_experts")
 class RoutedExperts(Part):
     NAMES = {"router": "router", "correction": "correction", "expert": "e{e}", "gate": "gate", "up": "up",
-             "down": "down", "shared": "shared"}
+             "down": "down", "shared": "shared", "shared_gate": "sg"}
 
     @classmethod
     def tensor_names(cls, params: Dict[str, Any]) -> Dict[str, str]:
@@ -65,6 +67,8 @@ class RoutedExperts(Part):
         if shared is not None:
             for name, spec in GatedMLP.weight_specs(shared).items():
                 specs[joined(n["shared"], name)] = spec
+            if params.get("shared_gate", False):
+                specs[joined(n["shared"], n["shared_gate"])] = TensorSpec((1, hidden), fan_in=hidden)
         return specs
 
     @classmethod
@@ -106,6 +110,9 @@ class RoutedExperts(Part):
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
         shared = self._shared_params(params)
         self.shared = GatedMLP(shared, joined(prefix, n["shared"]), build) if shared is not None else None
+        self.shared_gate = None
+        if self.shared is not None and params.get("shared_gate", False):
+            self.shared_gate = load.get(joined(joined(prefix, n["shared"]), n["shared_gate"])).reshape(-1).contiguous()
         self.score = params.get("score", "softmax")
         if self.score not in kernels.ROUTER_SCORES:
             raise ValueError(f"a router scores by {sorted(kernels.ROUTER_SCORES)}, not '{self.score}'")
@@ -153,4 +160,7 @@ class RoutedExperts(Part):
                                 activation=self.expert_activation, limit=self.limit)
             kernels.moe_down(x, act, self.w_down, idx, None if self.weight_on_input else weight, routed)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
+        if shared is not None and self.shared_gate is not None:
+            kernels.token_gate_add(x, self.shared_gate, shared, routed)
+            shared = None
         return routed, shared

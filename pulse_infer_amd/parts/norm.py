@@ -30,11 +30,13 @@ class RMSNorm(Part):
 
     records_cleanly = True
     takes_parts = True   # delta may be [parts, T, H] float32: the kernel adds the parts in order
+    takes_scale = True   # ``apply`` takes a factor on the update
 
     def apply(self, h: torch.Tensor, delta: Optional[torch.Tensor], out: torch.Tensor,
-              rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """out = norm(h + delta) * w; h keeps the sum unless rows are gathered."""
-        kernels.add_rmsnorm(h, delta, self.weight, self.eps, out, rows=rows, weight_offset=self.weight_offset)
+              rows: Optional[torch.Tensor] = None, delta_scale: float = 1.0) -> torch.Tensor:
+        """out = norm(h + delta_scale * delta) * w; h keeps the sum unless rows are gathered."""
+        kernels.add_rmsnorm(h, delta, self.weight, self.eps, out, rows=rows, weight_offset=self.weight_offset,
+                            delta_scale=delta_scale)
         return out
 
     def column_scale(self) -> Optional[torch.Tensor]:

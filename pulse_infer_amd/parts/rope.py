@@ -5,6 +5,7 @@ The reference rotates ADJACENT pairs (x[2i], x[2i+1])
 (x[i], x[i + rotary_dim/2]) instead.  Channels beyond ``rotary_dim`` pass unchanged.
 Once per step this part makes the cos/sin tables for the step's positions (angles in
 float64, tables float32); the mixer's fused kernel applies them to q and k.
+``scaling_factor`` f (default 1) divides every frequency by f ("linear scaling": position p turns like p / f).
 """
 from __future__ import annotations
 
@@ -45,7 +46,11 @@ class RotaryEmbedding(Part):
         self.pairing = PAIRINGS[pairing]
         half = self.rotary_dim // 2
         exponent = torch.arange(half, dtype=torch.float64) * (2.0 / self.rotary_dim)
-        self.inv_freq = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -exponent).to(build.device)
+        self.scaling_factor = float(params.get("scaling_factor", 1.0))
+        if not self.scaling_factor > 0:
+            raise ValueError(f"a rope scaling factor must be positive, got {self.scaling_factor}")
+        self.inv_freq = (torch.pow(torch.tensor(self.theta, dtype=torch.float64), -exponent)
+                         / self.scaling_factor).to(build.device)
         self.name = params.get("name", "rope")
 
     def prepare(self, ctx: StepContext) -> RotationTables:
