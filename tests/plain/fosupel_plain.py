@@ -115,7 +115,8 @@ def retention_walk(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: Lis
 
 
 def retention(x: torch.Tensor, w: Dict[str, torch.Tensor], p: str, m: Dict[str, Any], positions: List[int],
-              eps: float) -> torch.Tensor:
+              eps: float, sizes: Optional[list] = None) -> torch.Tensor:
+    """``sizes`` collects the root mean square of every head's output before it is divided by it, [T, heads]."""
     t, heads, d, dv = x.shape[0], m["heads"], m["dim"], m["vdim"]
     q = (x @ w[p + ".q"].T).view(t, heads, d)
     k = (x @ w[p + ".k"].T).view(t, heads, d)
@@ -125,13 +126,16 @@ def retention(x: torch.Tensor, w: Dict[str, torch.Tensor], p: str, m: Dict[str, 
         q = turn(q, positions, rot["base"], rot["dims"], "half")
         k = turn(k, positions, rot["base"], rot["dims"], "half")
     k = k * d ** -0.5
-    o = unit_rms(retention_walk(q, k, v, m["decay"]), eps)
+    o = retention_walk(q, k, v, m["decay"])
+    if sizes is not None:
+        sizes.append((o * o).mean(dim=-1).sqrt())
+    o = unit_rms(o, eps)
     return (o.reshape(t, heads * dv) * silu(x @ w[p + ".g"].T)) @ w[p + ".o"].T
 
 
-def parallel_mixer(x, w, p, m, positions, eps):
+def parallel_mixer(x, w, p, m, positions, eps, sizes=None):
     return (m["left_scale"] * talking_window_attention(x, w, p + ".left", m["left"], positions)
-            + m["right_scale"] * retention(x, w, p + ".right", m["right"], positions, eps))
+            + m["right_scale"] * retention(x, w, p + ".right", m["right"], positions, eps, sizes))
 
 
 def latent_attention(x: torch.Tensor, w: Dict[str, torch.Tensor], p: str, m: Dict[str, Any], positions: List[int],
@@ -196,8 +200,21 @@ def layer_order(cfg: Dict[str, Any]) -> List[tuple]:
     return out + [(i, None) for i in range(loop["stop"], n)]
 
 
+def fragile_positions(cfg: Dict[str, Any], w: Dict[str, torch.Tensor], tokens: List[int], below: float = 0.1) -> set:
+    """Positions at which some retention head's output, which is divided by its own root mean square, is smaller than
+    ``below`` times what that head usually gives: the division multiplies whatever rounding left in it by as much, in
+    any arithmetic, so no bound that holds elsewhere says anything there."""
+    sizes: List[torch.Tensor] = []
+    forward(cfg, w, tokens, sizes=sizes)
+    out: set = set()
+    for rms in sizes:
+        usual = rms.median(dim=0, keepdim=True).values
+        out |= set((rms < below * usual).any(dim=1).nonzero().flatten().tolist())
+    return out
+
+
 def forward(cfg: Dict[str, Any], w: Dict[str, torch.Tensor], tokens: List[int], residuals: Optional[list] = None,
-            margins: Optional[list] = None) -> torch.Tensor:
+            margins: Optional[list] = None, sizes: Optional[list] = None) -> torch.Tensor:
     """Logits [T, vocab] of one sequence; ``residuals`` collects the stream after every layer run."""
     w = {k: v.to(DT) for k, v in w.items()}
     eps, mult = cfg["norm"]["eps"], cfg.get("residual_mult", 1.0)
@@ -209,7 +226,7 @@ def forward(cfg: Dict[str, Any], w: Dict[str, torch.Tensor], tokens: List[int], 
             x = x + w["loop.step"][step]
         n = unit_rms(x, eps) * w[p + ".norm1"]
         if layer["type"] == "parallel":
-            x = x + mult * parallel_mixer(n, w, p + ".mix", layer["mixer"], positions, eps)
+            x = x + mult * parallel_mixer(n, w, p + ".mix", layer["mixer"], positions, eps, sizes)
         elif layer["type"] == "latent_attention":
             x = x + mult * latent_attention(n, w, p + ".mix", layer["mixer"], positions, eps)
         else:
@@ -238,3 +255,37 @@ def load_folder(path: str):
         if name.endswith(".safetensors"):
             w.update(load_file(os.path.join(path, name)))
     return cfg, w
+
+
+class PlainFosupel:
+    """The functions above behind the few calls the tests make."""
+
+    def __init__(self, cfg: Dict[str, Any], weights: Dict[str, torch.Tensor]):
+        self.cfg = cfg
+        self.w = {k: v.to(DT) for k, v in weights.items()}
+
+    @classmethod
+    def from_folder(cls, path: str) -> "PlainFosupel":
+        return cls(*load_folder(path))
+
+    def logits(self, ids: List[int]) -> torch.Tensor:
+        return forward(self.cfg, self.w, list(ids))
+
+    def residuals(self, ids: List[int]) -> List[torch.Tensor]:
+        out: List[torch.Tensor] = []
+        forward(self.cfg, self.w, list(ids), residuals=out)
+        return out
+
+    def router_margins(self, ids: List[int]) -> torch.Tensor:
+        return router_margins(self.cfg, self.w, list(ids))
+
+    def fragile_positions(self, ids: List[int]) -> set:
+        return fragile_positions(self.cfg, self.w, list(ids))
+
+    def greedy(self, prompt: List[int], new: int) -> List[int]:
+        ids, out = list(prompt), []
+        for _ in range(new):
+            token = int(self.logits(ids)[-1].argmax())
+            out.append(token)
+            ids.append(token)
+        return out
