@@ -55,7 +55,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
     p.add_argument("--model", choices=sorted(SHAPES), default="8b", help="layer sizes: Qwen3-8B (the default), 14B or 32B")
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has, if memory or time needs it")
-    p.add_argument("--workload", choices=["decode", "serving", "long-prompt", "dirozen", "kesovik", "tipidra"], default="decode",
+    p.add_argument("--workload", choices=["decode", "serving", "long-prompt", "dirozen", "kesovik", "tipidra", "fosupel"], default="decode",
                    help="decode: fixed batch at a fixed context; serving: continuous batching of requests with "
                         "seeded prompt lengths, chunked prefill mixed with decoding; long-prompt: one prompt of "
                         "--prompt-tokens tokens in portions of --chunk tokens; dirozen / kesovik: decoding and prefill of "
@@ -269,6 +269,30 @@ def tipidra_layers(size, layers):
     return [turn[i % len(turn)] for i in range(layers)]
 
 
+def fosupel_layers(size, layers):
+    """Fosupel layers at the comparison's sizes, in turn: two mixers side by side (attention over a window of 1,024
+    tokens with 4 kept first tokens, sinks and mixed heads, a rotation on half of a head with scaled frequencies, beside
+    retention with half as many heads) with a dense feed-forward; the same with routed experts; latent attention (heads
+    as Qwen3's, a latent row of 512 values and a turned part of 64) with a dense feed-forward; the first pair with
+    routed experts again.  The routed feed-forward has 16 experts an eighth as wide as the dense one, 4 chosen a token,
+    and a gated shared expert a quarter as wide."""
+    dim = size["dim"]
+    left = {"dim": dim, "heads": size["heads"], "kv_heads": size["kv_heads"], "mask": {"keep_first": 4, "size": 1024},
+            "rot": {"base": 1e6, "dims": dim // 2, "scaling": {"factor": 2.0}}, "scale": dim ** -0.5, "vdim": dim}
+    heads = size["heads"] // 2
+    right = {"decay": [1.0 - 2.0 ** -(5 + 8.0 * h / heads) for h in range(heads)], "dim": dim, "heads": heads,
+             "rot": {"base": 1e6, "dims": dim // 2}, "vdim": dim}
+    both = {"left": left, "left_scale": 0.9, "right": right, "right_scale": 1.2}
+    latent = {"dim": dim, "heads": size["heads"], "kv_rank": 512, "rot": {"base": 1e6, "dims": 64}, "rot_dim": 64,
+              "scale": (dim + 64) ** -0.5, "vdim": dim}
+    dense = {"ff": size["ff"], "kind": "dense"}
+    routed = {"expert": {"ff": size["ff"] // 8}, "kind": "moe", "router": {"experts": 16, "top": 4},
+              "shared": {"ff": size["ff"] // 4}}
+    turn = [{"type": "parallel", "mixer": both, "mlp": dense}, {"type": "parallel", "mixer": both, "mlp": routed},
+            {"type": "latent_attention", "mixer": latent, "mlp": dense}, {"type": "parallel", "mixer": both, "mlp": routed}]
+    return [turn[i % len(turn)] for i in range(layers)]
+
+
 def dirozen_compare(args, design: str = "dirozen") -> int:
     """Dirozen (or, with ``design`` "kesovik", Kesovik) beside Qwen3 layers of equal sizes (random weights, ``--compare-layers`` layers, a vocabulary of
     32,000): decoding at batch 1 / 8 / 32 with contexts ending at ``--context`` and a prompt of ``--prefill-tokens``
@@ -277,7 +301,7 @@ def dirozen_compare(args, design: str = "dirozen") -> int:
     line."""
     import torch
 
-    from pulse_infer_amd.config import DirozenConfig, KesovikConfig, Qwen3Config, TipidraConfig
+    from pulse_infer_amd.config import DirozenConfig, FosupelConfig, KesovikConfig, Qwen3Config, TipidraConfig
     from pulse_infer_amd.engine.engine import ContinuousBatchEngine
     from pulse_infer_amd.engine.runner import StepEntry
     from pulse_infer_amd.models.causal_lm import expected_tensors
@@ -307,7 +331,7 @@ def dirozen_compare(args, design: str = "dirozen") -> int:
                  "mlp": {"ff": size["ff"], "kind": "dense"}}
         dirozen = DirozenConfig.from_dict({"architecture": "Dirozen", "vocab": vocab, "width": size["width"],
                                            "norm": {"eps": 1e-6}, "layers": [entry] * layers}, "<bench>")
-        if design in ("kesovik", "tipidra"):
+        if design in ("kesovik", "tipidra", "fosupel"):
             kesovik = KesovikConfig.from_dict({
                 "architecture": "Kesovik", "vocab": vocab, "width": size["width"], "norm": {"eps": 1e-6},
                 "embedding": {"scale": 1.0}, "postln_alpha": 2.0, "logit_softcap": 30.0,
@@ -318,6 +342,11 @@ def dirozen_compare(args, design: str = "dirozen") -> int:
                     "embedding": {"scale": 1.0}, "logit_softcap": 30.0, "streams": 4,
                     "layers": tipidra_layers(size, layers)}, "<bench>")
                 return {"tipidra": tipidra, "kesovik": kesovik, "qwen3": qwen}
+            if design == "fosupel":
+                fosupel = FosupelConfig.from_dict({
+                    "architecture": "Fosupel", "vocab": vocab, "width": size["width"], "norm": {"eps": 1e-6},
+                    "residual_mult": 0.5, "logit_softcap": 30.0, "layers": fosupel_layers(size, layers)}, "<bench>")
+                return {"fosupel": fosupel, "kesovik": kesovik, "qwen3": qwen}
             return {"kesovik": kesovik, "qwen3": qwen}
         return {"dirozen": dirozen, "qwen3": qwen}
 
@@ -402,7 +431,7 @@ def dirozen_compare(args, design: str = "dirozen") -> int:
         torch.cuda.empty_cache()
         return out
 
-    record = {"metric": f"{design}_beside_{'kesovik_and_' if design == 'tipidra' else ''}qwen3_layers", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype,
+    record = {"metric": f"{design}_beside_{'kesovik_and_' if design in ('tipidra', 'fosupel') else ''}qwen3_layers", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype,
               "data": "synthetic", "layers": layers, "vocab": vocab, "context": args.context, "sizes": {}}
     for name, size in DIROZEN_SIZES.items():
         if name not in args.compare_sizes.split(","):
@@ -421,7 +450,7 @@ def dirozen_compare(args, design: str = "dirozen") -> int:
 
 def main() -> int:
     args = parse_args()
-    if args.workload in ("kesovik", "tipidra"):
+    if args.workload in ("kesovik", "tipidra", "fosupel"):
         return dirozen_compare(args, args.workload)
     if args.workload == "dirozen":
         if args.gpus != 1:

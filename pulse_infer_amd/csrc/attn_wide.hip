@@ -1,0 +1,263 @@
+// Paged attention on the matrix cores for query heads that gather WIDE values: the values of every kv head side by
+// side (a caller that mixes the heads' weights afterwards) or one wide latent row shared by all heads; with a window
+// that keeps a request's first tokens, and sinks.  bfloat16 operands, float32 everything else, float32 results.
+//
+// An item is 16 rows: `hp` query heads of one kv head for 16 / hp consecutive tokens of one request (a decoded token
+// is an item of its group's heads alone).  A workgroup takes an item and a chunk of up to 256 value channels; its four
+// wavefronts share the item's keys out in steps of 32 and meet in LDS at the end.  Per step and wavefront:
+//
+//   S^T = K Q^T      two tiles of 16 keys x 16 rows (v_mfma_f32_16x16x32_bf16 over the head's channels): a lane then
+//                    holds, for ITS row (lane % 16), the scores of keys 4 (lane / 16) + i of both tiles;
+//   softmax          running maximum and sum per row (a row's lanes meet by two shuffles), scores never leave registers;
+//   O^T += V^T P^T   the lane's eight weights ARE its share of the P^T operand if the step's 32 keys are taken in the
+//                    order tile 0 keys 4g..4g+3, tile 1 keys 4g..4g+3 (g = lane / 16), so the V^T operand is read in
+//                    that order: two 8-byte loads from the page's channel-major values.
+//
+// Keys come straight from the pages.  The visible keys of an item are the kept first tokens (rounded up to whole
+// 16-key tiles) and the tiles from the one that holds the first row's window start to the last row's position; what a
+// row must not see inside them is masked by its own position.  Values of keys behind the item's last position have
+// never been written and are cleared in the operand (a weight of zero times whatever lies there must stay zero).
+#include "common.h"
+
+#include <math.h>
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+
+constexpr int CHUNK_TILES = 16;             // channel tiles of 16 a workgroup accumulates
+constexpr int CHUNK = 16 * CHUNK_TILES;
+
+struct WideArgs {
+    int nq, nkv, d;       // d: stored channels of a head (keys and values alike)
+    int w;                // value channels a query head gathers: nkv * d with all_values, else d
+    int wv;               // of which are computed (a multiple of 16)
+    int all_values, hp;
+    int64_t q_stride, o_stride;
+    int page_size, num_pages, bt_width;
+    float scale, cap;
+    int window, keep_first;
+};
+
+__device__ __forceinline__ bf16x8 zeros8() {
+    return __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+}
+
+__global__ __launch_bounds__(256) void attn_wide_kernel(const bf16_t* __restrict__ q, float* __restrict__ out,
+                                                        const bf16_t* __restrict__ kcache,
+                                                        const bf16_t* __restrict__ vcache,
+                                                        const int* __restrict__ positions,
+                                                        const int* __restrict__ token_entry,
+                                                        const int* __restrict__ block_table,
+                                                        const int* __restrict__ items, const float* __restrict__ sink,
+                                                        WideArgs a) {
+    __shared__ float red[3][CHUNK_TILES][PULSE_WAVE][4];
+    __shared__ float ml[4][16][2];
+    const int* it = items + 4 * blockIdx.x;
+    const int t0 = it[0], nt = it[1], head0 = it[2], nh = it[3];
+    const int chunk0 = blockIdx.y * CHUNK;
+    const int tiles = min(CHUNK_TILES, (a.wv - chunk0) / 16);
+    const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
+    const int r = lane % 16, g = lane / 16;
+    const int ti = r / a.hp, hi = r % a.hp;
+    const bool valid = ti < nt && hi < nh;
+    const int tok = t0 + (valid ? ti : 0), head = head0 + (valid ? hi : 0);
+    const int pos = positions[tok];
+    const int kvh = head0 / (a.nq / a.nkv);
+    const int* bt = block_table + static_cast<int64_t>(token_entry[t0]) * a.bt_width;
+    const int pos_first = positions[t0], pos_last = positions[t0 + nt - 1];
+    const int lo = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
+    const int lo16 = lo & ~15;
+    const int nfirst = a.window > 0 ? min((a.keep_first + 15) & ~15, lo16) : 0;
+    const int total = nfirst + pos_last + 1 - lo16;
+    const int nsteps = (total + 31) / 32;
+    const int d = a.d;
+    const bf16_t* qrow = q + static_cast<int64_t>(tok) * a.q_stride + static_cast<int64_t>(head) * d;
+
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4 acc[CHUNK_TILES];
+#pragma unroll
+    for (int c = 0; c < CHUNK_TILES; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int step = wave; step < nsteps; step += 4) {
+        int page[2], off[2], jbase[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int ub = step * 32 + 16 * t;
+            const int jb = ub < nfirst ? ub : lo16 + ub - nfirst;
+            const int pi = jb / a.page_size;
+            const int p = (ub < total && pi < a.bt_width) ? bt[pi] : -1;
+            page[t] = (p >= 0 && p < a.num_pages) ? p : -1;
+            off[t] = jb % a.page_size;
+            jbase[t] = jb;
+        }
+        // S^T: keys x rows
+        f32x4 s[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+        const bf16_t* krow[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+            krow[t] = page[t] >= 0 ? kcache + ((static_cast<int64_t>(page[t]) * a.nkv + kvh) * a.page_size + off[t] + r) * d
+                                   : nullptr;
+        for (int e0 = 0; e0 < d; e0 += 32) {
+            const int e = e0 + 8 * g;
+            const bool in = e < d;
+            const bf16x8 qb = in ? *reinterpret_cast<const bf16x8*>(qrow + e) : zeros8();
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const bf16x8 ka = (in && krow[t]) ? *reinterpret_cast<const bf16x8*>(krow[t] + e) : zeros8();
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb, s[t], 0, 0, 0);
+            }
+        }
+        // this row's scores of keys jbase[t] + 4 g + i
+        float v[2][4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = jbase[t] + 4 * g + i;
+                const bool seen = valid && page[t] >= 0 && j <= pos && (a.window == 0 || pos - j < a.window || j < a.keep_first);
+                float x = s[t][i] * a.scale;
+                if (a.cap > 0.f) x = a.cap * tanhf(x / a.cap);
+                v[t][i] = seen ? x : -INFINITY;
+                mx = fmaxf(mx, v[t][i]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, PULSE_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, PULSE_WAVE));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = (m_new == -INFINITY) ? 1.f : expf(m_run - m_new);
+        float p[2][4], sum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p[t][i] = (v[t][i] == -INFINITY) ? 0.f : expf(v[t][i] - m_new);
+                sum += p[t][i];
+            }
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+        bf16x8 pb;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pb[4 * t + i] = static_cast<__bf16>(p[t][i]);
+        // O^T += V^T P^T, channel tile by channel tile
+        bool written[2][4];   // keys of the operand that have ever been stored
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) written[t][i] = page[t] >= 0 && jbase[t] + 4 * g + i <= pos_last;
+#pragma unroll
+        for (int c = 0; c < CHUNK_TILES; ++c) {
+            if (c < tiles) {
+                acc[c] *= alpha;
+                const int ch = chunk0 + 16 * c + r;
+                const int vh = a.all_values ? ch / d : kvh;
+                const int e = a.all_values ? ch % d : ch;
+                u32x4 raw = {0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    if (page[t] >= 0) {
+                        const u32x2 two = *reinterpret_cast<const u32x2*>(
+                            vcache + ((static_cast<int64_t>(page[t]) * a.nkv + vh) * d + e) * a.page_size + off[t] + 4 * g);
+                        raw[2 * t] = two[0];
+                        raw[2 * t + 1] = two[1];
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    if (!written[t][0]) raw[2 * t] &= 0xFFFF0000u;
+                    if (!written[t][1]) raw[2 * t] &= 0x0000FFFFu;
+                    if (!written[t][2]) raw[2 * t + 1] &= 0xFFFF0000u;
+                    if (!written[t][3]) raw[2 * t + 1] &= 0x0000FFFFu;
+                }
+                acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, raw), pb, acc[c], 0, 0, 0);
+            }
+        }
+    }
+    // a row's sum over the four lanes that share it; then the four wavefronts meet
+    l_run += __shfl_xor(l_run, 16, PULSE_WAVE);
+    l_run += __shfl_xor(l_run, 32, PULSE_WAVE);
+    if (g == 0) { ml[wave][r][0] = m_run; ml[wave][r][1] = l_run; }
+    __syncthreads();
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) m_all = fmaxf(m_all, ml[w][r][0]);
+    float l_all = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) l_all += (ml[w][r][0] == -INFINITY) ? 0.f : ml[w][r][1] * expf(ml[w][r][0] - m_all);
+    const float mine = (m_run == -INFINITY) ? 0.f : expf(m_run - m_all);
+#pragma unroll
+    for (int c = 0; c < CHUNK_TILES; ++c) {
+        if (c < tiles) {
+            acc[c] *= mine;
+            if (wave > 0) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) red[wave - 1][c][lane][i] = acc[c][i];
+            }
+        }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    // a sink is one more term of the softmax's denominator, exp(sink[h]), with no key and no value
+    float scale_out = 1.f;
+    if (sink) {
+        const float sk = sink[head];
+        if (m_all == -INFINITY) l_all = 1.f;
+        else if (sk > m_all) { scale_out = expf(m_all - sk); l_all = l_all * scale_out + 1.f; }
+        else l_all += expf(sk - m_all);
+    }
+    const float inv = l_all > 0.f ? scale_out / l_all : 0.f;
+    if (!valid) return;
+    float* orow = out + static_cast<int64_t>(tok) * a.o_stride + static_cast<int64_t>(head) * a.w + chunk0;
+#pragma unroll
+    for (int c = 0; c < CHUNK_TILES; ++c) {
+        if (c < tiles) {
+            f32x4 sum = acc[c];
+#pragma unroll
+            for (int w = 0; w < 3; ++w)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sum[i] += red[w][c][lane][i];
+            *reinterpret_cast<f32x4*>(orow + 16 * c + 4 * g) = sum * inv;
+        }
+    }
+}
+
+}  // namespace
+
+// q [tokens, q_stride] bfloat16: head h's query at h * d.  out float32 [tokens, o_stride]: head h's result at h * w,
+// w = nkv * d with all_values (value head c at c * d) else d; channels 0 .. wv - 1 of it are written.  items int32
+// [n_items, 4]: first token, tokens, first head, heads; row r of an item is token r / hp, head r % hp.  kcache
+// [pages, nkv, page, d], vcache [pages, nkv, d, page] bfloat16, page_size a multiple of 16, d a multiple of 16.
+extern "C" int pulse_attn_wide(const void* q, int64_t q_stride, float* out, int64_t o_stride, const void* kcache,
+                               const void* vcache, const int* positions, const int* token_entry, const int* block_table,
+                               int bt_width, const int* items, int n_items, int hp, int nq, int nkv, int d, int wv,
+                               int all_values, int page_size, int num_pages, float scale, int window, int keep_first,
+                               const float* sink, float softcap, hipStream_t stream) {
+    PULSE_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0 && d > 0 && d % 16 == 0, "attn_wide: bad head sizes");
+    PULSE_REQUIRE(page_size > 0 && page_size % 16 == 0 && num_pages > 0 && bt_width > 0, "attn_wide: pages must hold a multiple of 16 keys");
+    const int w = all_values ? nkv * d : d;
+    PULSE_REQUIRE(wv > 0 && wv % 16 == 0 && wv <= w, "attn_wide: %d of %d value channels", wv, w);
+    PULSE_REQUIRE(hp >= 1 && hp <= 16 && n_items >= 0, "attn_wide: bad items");
+    PULSE_REQUIRE(window >= 0 && keep_first >= 0 && softcap >= 0.f, "attn_wide: bad window, kept keys or score cap");
+    PULSE_REQUIRE(q_stride >= static_cast<int64_t>(nq) * d && o_stride >= static_cast<int64_t>(nq) * w && o_stride % 4 == 0 &&
+                  q_stride % 8 == 0, "attn_wide: row strides too small or unaligned");
+    PULSE_REQUIRE(q && out && kcache && vcache && positions && token_entry && block_table && items, "attn_wide: null pointer");
+    PULSE_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(kcache) % 16 == 0 && reinterpret_cast<uintptr_t>(vcache) % 16 == 0,
+                  "attn_wide: operands must be 16-byte aligned");
+    if (n_items == 0) return 0;
+    WideArgs a;
+    a.nq = nq; a.nkv = nkv; a.d = d; a.w = w; a.wv = wv; a.all_values = all_values ? 1 : 0; a.hp = hp;
+    a.q_stride = q_stride; a.o_stride = o_stride; a.page_size = page_size; a.num_pages = num_pages; a.bt_width = bt_width;
+    a.scale = scale; a.cap = softcap; a.window = window; a.keep_first = window > 0 ? keep_first : 0;
+    const dim3 grid(n_items, (wv + CHUNK - 1) / CHUNK);
+    hipLaunchKernelGGL(attn_wide_kernel, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(q), out,
+                       static_cast<const bf16_t*>(kcache), static_cast<const bf16_t*>(vcache), positions, token_entry,
+                       block_table, items, sink, a);
+    PULSE_LAUNCH_CHECK("attn_wide");
+    return 0;
+}

@@ -534,6 +534,60 @@ def attn_generic(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, 
          _i32(1 if all_values else 0), _i32(1 if out.dtype == torch.float32 else 0), _stream())
 
 
+def attn_wide_takes(q: torch.Tensor, kcache: torch.Tensor, d: int) -> bool:
+    """Whether ``attn_wide`` takes these operands: bfloat16 queries and pages, pages of a multiple of 16 keys, heads
+    stored a multiple of 16 channels wide."""
+    return (q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and kcache.dim() == 4
+            and kcache.shape[2] % 16 == 0 and d % 16 == 0)
+
+
+def attn_wide_items(entries, nq: int, nkv: int):
+    """The work list of ``attn_wide`` for a step's entries (anything with ``first_row`` and ``count``): items of 16
+    rows, ``hp`` heads of one kv head for 16 // hp consecutive tokens of one entry.  Returns (flat list of
+    quadruples first token, tokens, first head, heads; hp)."""
+    group = nq // nkv
+    hp = min(group, 16)
+    tp = 16 // hp
+    flat = []
+    for e in entries:
+        for t in range(0, e.count, tp):
+            nt = min(tp, e.count - t)
+            for a in range(nkv):
+                for hb in range(0, group, hp):
+                    flat.extend((e.first_row + t, nt, a * group + hb, min(hp, group - hb)))
+    return flat, hp
+
+
+def attn_wide(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, wv: int, all_values: bool,
+              kcache: torch.Tensor, vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor,
+              block_table: torch.Tensor, items: torch.Tensor, hp: int, scale: float, window: int = 0,
+              keep_first: int = 0, sink: Optional[torch.Tensor] = None, softcap: float = 0.0) -> None:
+    """Paged attention on the matrix cores for heads that gather wide values: with ``all_values`` every query head's
+    weights on the values of all kv heads (out float32 [T, nq * nkv * d], as ``attn_generic`` leaves it), else on its
+    own kv head's (out float32 [T, nq * d]); of a head's channels the first ``wv`` (a multiple of 16) are written.
+    Window, kept first keys, sinks and score cap as for ``attn_generic``."""
+    _gpu("attn_wide", q, out, kcache, vcache, positions, token_entry, block_table, items, sink)
+    tokens = q.shape[0]
+    _need(attn_wide_takes(q, kcache, d), "attn_wide: bfloat16 operands, pages of a multiple of 16 keys, d % 16 == 0")
+    width = nq * d * (nkv if all_values else 1)
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * d, "attn_wide: q too narrow")
+    _need(out.dtype == torch.float32 and out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == tokens
+          and out.shape[1] >= width, f"attn_wide: out must be float32 [{tokens}, {width}]")
+    pages, page_size = _check_cache("attn_wide", kcache, vcache, nkv, d)
+    _int_vec("attn_wide: positions", positions, tokens)
+    _int_vec("attn_wide: token_entry", token_entry, tokens)
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+          "attn_wide: block_table must be contiguous int32 [entries, width]")
+    _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() % 4 == 0, "attn_wide: items are int32 quadruples")
+    if sink is not None:
+        _need(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == nq, f"attn_wide: the sinks must be float32 [{nq}]")
+    call("pulse_attn_wide", _ptr(q), _i64(q.stride(0) if tokens > 1 else q.shape[1]), _ptr(out),
+         _i64(out.stride(0) if tokens > 1 else out.shape[1]), _ptr(kcache), _ptr(vcache), _ptr(positions), _ptr(token_entry),
+         _ptr(block_table), _i32(block_table.shape[1]), _ptr(items), _i32(items.numel() // 4), _i32(hp), _i32(nq), _i32(nkv),
+         _i32(d), _i32(wv), _i32(1 if all_values else 0), _i32(page_size), _i32(pages), _f32(scale), _i32(window),
+         _i32(keep_first), _ptr(sink), _f32(softcap), _stream())
+
+
 def head_mix(x: torch.Tensor, mix: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, d: int, dv: int,
              out_d: int, scale: float = 1.0) -> None:
     """out[t, h, e] = scale * sum_g mix[h, g] * x[t, g, h // (heads // kv_heads), e] for e < dv, zero for dv <= e <

@@ -13,8 +13,9 @@ projection and whose sigmoid the attention kernels apply as they store; ``score_
 ``attention``; ``keep_first`` (with a window): a request's first ``keep_first`` tokens stay visible below the window,
 at their true positions; ``talk``: the heads' attention weights are mixed before they meet the values, weight_h <-
 sum_g T[h, g] weight_g with T the tensor ``talk`` [heads, heads] (a sink's share is not mixed); head h applies its
-mixed weights to the values of its own kv head.  Both run on the generic attention kernel: with ``talk`` it leaves
-every head's weights applied to the values of every kv head, in float32, and ``pulse_head_mix`` forms the sums.
+mixed weights to the values of its own kv head.  Both run on ``pulse_attn_wide`` (bfloat16, the matrix cores) or the
+generic attention kernel: with ``talk`` either leaves every head's weights applied to the values of every kv head, in
+float32, and ``pulse_head_mix`` forms the sums.
 
 Keys and values are stored with one width D = max(head_dim, value_dim) rounded up to a multiple of 16, the missing
 channels as zeros: zero key channels add nothing to a score, and zero value channels come out as zeros, which meet
@@ -190,18 +191,44 @@ class RowPreparedAttention(PagedAttention):
             self.attend(q, out, ctx, cache, table, gate=gate)
             return
         window = int(self.window) if self.window is not None else 0
-        if not self.talks:
+        wide = (self.options.get("attention", "auto") != "generic" and gate is None
+                and kernels.attn_wide_takes(q, cache.keys, self.d))
+        if not self.talks and not wide:
             kernels.attn_generic(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
                                  ctx.token_entry, table, self.scale, window, gate=gate, gate_width=self.gate_width,
                                  sink=self.sink, softcap=self.score_cap, keep_first=self.keep_first)
             return
-        # every head's weights on every kv head's values, then the sums over heads that the mixing matrix asks for
-        # (the branch's factor is already in the stored values)
-        each = ws.buffer("attention_rows.each", tokens, self.nq * self.nkv * self.d, torch.float32)
-        kernels.attn_generic(q, each, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
-                             ctx.token_entry, table, self.scale, window, sink=self.sink, softcap=self.score_cap,
-                             keep_first=self.keep_first, all_values=True)
-        kernels.head_mix(each, self.talk, out, self.nq, self.nkv, self.d, self.v_dim, self.d)
+        # float32 rows first: with mixed heads every head's weights on every kv head's values, then the sums over heads
+        # that the mixing matrix asks for; without, the rows as they are (the branch's factor is in the stored values)
+        width = self.nq * self.d * (self.nkv if self.talks else 1)
+        each = ws.buffer("attention_rows.each", tokens, width, torch.float32)
+        if wide:
+            items, hp = self._wide_items(ctx)
+            kernels.attn_wide(q, each, self.nq, self.nkv, self.d, self.nkv * self.d if self.talks else self.d, self.talks,
+                              cache.keys, cache.values, ctx.positions, ctx.token_entry, table, items, hp, self.scale,
+                              window, self.keep_first, self.sink, self.score_cap)
+        else:
+            kernels.attn_generic(q, each, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
+                                 ctx.token_entry, table, self.scale, window, sink=self.sink, softcap=self.score_cap,
+                                 keep_first=self.keep_first, all_values=True)
+        if self.talks:
+            kernels.head_mix(each, self.talk, out, self.nq, self.nkv, self.d, self.v_dim, self.d)
+        else:
+            kernels.head_mix(each, self._identity(each.device), out, self.nq, 1, self.d, self.v_dim, self.d)
+
+    def _wide_items(self, ctx: StepContext):
+        """The work list of ``attn_wide`` for this step (it depends on the step's shape alone; every layer with these
+        head counts shares it)."""
+        key = f"static:attention_rows.wide_items:{self.nq}:{self.nkv}"
+        if key not in ctx.extras:
+            flat, hp = kernels.attn_wide_items(ctx.entries, self.nq, self.nkv)
+            ctx.extras[key] = (ctx.to_device(flat), hp)
+        return ctx.extras[key]
+
+    def _identity(self, device) -> torch.Tensor:
+        if getattr(self, "_eye", None) is None:
+            self._eye = torch.eye(self.nq, dtype=torch.float32, device=device)
+        return self._eye
 
     def decodes_from_raw(self, ctx, cache, qkv, tables) -> bool:
         return False

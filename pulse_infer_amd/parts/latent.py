@@ -144,10 +144,24 @@ class LatentAttention(PagedAttention):
                             self.rank, self.d, self.eps, write=cache.writable)
         kernels.latent_absorb(y, 0, self.plain_dim + self.rot_dim, self.w_uk, q, self.d, self.nq, self.plain_dim,
                               self.rank)
-        # the weighted latent rows: float32 from the generic kernel, the activations' type from the matrix cores
-        kind = self.act_dtype if self.uses_matrix_cores(q, cache) else torch.float32
-        o = ws.buffer("latent.rows", tokens, self.nq * self.d, kind)
-        self.attend(q, o, ctx, cache, table)
+        # the weighted latent rows: from the matrix-core kernels of ``attention`` where they are compiled for rows this
+        # wide (the activations' type), else in float32 from the matrix-core kernel for wide values or the generic one
+        if self.uses_matrix_cores(q, cache):
+            o = ws.buffer("latent.rows", tokens, self.nq * self.d, self.act_dtype)
+            self.attend(q, o, ctx, cache, table)
+        elif self.options.get("attention", "auto") != "generic" and kernels.attn_wide_takes(q, cache.keys, self.d):
+            o = ws.buffer("latent.rows", tokens, self.nq * self.d, torch.float32)
+            key = f"static:latent.wide_items:{self.nq}"
+            if key not in ctx.extras:
+                flat, hp = kernels.attn_wide_items(ctx.entries, self.nq, 1)
+                ctx.extras[key] = (ctx.to_device(flat), hp)
+            items, hp = ctx.extras[key]
+            kernels.attn_wide(q, o, self.nq, 1, self.d, (self.rank + 15) // 16 * 16, False, cache.keys, cache.values,
+                              ctx.positions, ctx.token_entry, table, items, hp, self.scale, 0, 0, self.sink, self.score_cap)
+        else:
+            o = ws.buffer("latent.rows", tokens, self.nq * self.d, torch.float32)
+            kernels.attn_generic(q, o, self.nq, 1, self.d, cache.keys, cache.values, ctx.positions, ctx.token_entry,
+                                 table, self.scale, 0, sink=self.sink, softcap=self.score_cap)
         gate = y[:, self.gate_col0:self.gate_col0 + self.nq * self.v_dim] if self.gated else None
         kernels.latent_expand(o, self.d, self.w_uv, gate, out, self.nq, self.v_dim, self.rank, self.out_scale)
 

@@ -200,17 +200,20 @@ def layer_order(cfg: Dict[str, Any]) -> List[tuple]:
     return out + [(i, None) for i in range(loop["stop"], n)]
 
 
-def fragile_positions(cfg: Dict[str, Any], w: Dict[str, torch.Tensor], tokens: List[int], below: float = 0.1) -> set:
-    """Positions at which some retention head's output, which is divided by its own root mean square, is smaller than
-    ``below`` times what that head usually gives: the division multiplies whatever rounding left in it by as much, in
-    any arithmetic, so no bound that holds elsewhere says anything there."""
-    sizes: List[torch.Tensor] = []
-    forward(cfg, w, tokens, sizes=sizes)
-    out: set = set()
-    for rms in sizes:
-        usual = rms.median(dim=0, keepdim=True).values
-        out |= set((rms < below * usual).any(dim=1).nonzero().flatten().tolist())
-    return out
+def fragile_positions(cfg: Dict[str, Any], w: Dict[str, torch.Tensor], tokens: List[int], above: float = 4.0) -> set:
+    """Positions whose logits hang on cancellations: where these same equations evaluated in float32 stray from their
+    float64 values ``above`` times further than at the median position.  (A retention head's output is divided by its
+    own root mean square; where that output is small by chance, the division multiplies whatever rounding left in it,
+    in any arithmetic, and no bound that holds elsewhere says anything there.)"""
+    global DT
+    exact = forward(cfg, w, tokens)
+    DT = torch.float32
+    try:
+        rough = forward(cfg, w, tokens).to(torch.float64)
+    finally:
+        DT = torch.float64
+    err = (rough - exact).abs().max(dim=1).values
+    return set((err > above * err.median()).nonzero().flatten().tolist())
 
 
 def forward(cfg: Dict[str, Any], w: Dict[str, torch.Tensor], tokens: List[int], residuals: Optional[list] = None,
