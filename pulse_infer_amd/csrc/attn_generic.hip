@@ -175,7 +175,8 @@ extern "C" int pulse_attn_generic_ex(const void* q, int64_t q_stride, void* out,
     const int width = all_values ? nkv * d : d;
     PULSE_REQUIRE(tokens >= 0 && nq > 0 && nkv > 0 && d > 0, "attn_generic: bad sizes");
     PULSE_REQUIRE(nq % nkv == 0, "attn_generic: %d query heads are not a multiple of %d kv heads", nq, nkv);
-    PULSE_REQUIRE(width <= PULSE_WAVE * 32, "attn_generic: %d value channels a query head exceed %d", width, PULSE_WAVE * 32);
+    PULSE_REQUIRE(width <= PULSE_WAVE * 32, "attn_generic: head_dim %d gives %d value channels a query head, more than %d", d,
+                  width, PULSE_WAVE * 32);
     PULSE_REQUIRE(nq < 65536, "attn_generic: at most 65535 query heads, got %d", nq);
     PULSE_REQUIRE(page_size > 0 && num_pages > 0 && bt_width > 0, "attn_generic: bad cache geometry");
     PULSE_REQUIRE(window >= 0 && keep_first >= 0, "attn_generic: negative window or kept keys");

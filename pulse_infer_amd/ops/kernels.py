@@ -585,7 +585,7 @@ def attn_wide(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, wv:
          _i64(out.stride(0) if tokens > 1 else out.shape[1]), _ptr(kcache), _ptr(vcache), _ptr(positions), _ptr(token_entry),
          _ptr(block_table), _i32(block_table.shape[1]), _ptr(items), _i32(items.numel() // 4), _i32(hp), _i32(nq), _i32(nkv),
          _i32(d), _i32(wv), _i32(1 if all_values else 0), _i32(page_size), _i32(pages), _f32(scale), _i32(window),
-         _i32(keep_first), _ptr(sink), _f32(softcap), _stream())
+         _i32(keep_first), _ptr(sink), _f32(softcap), _stream(), label=f"d={d} values={wv}")
 
 
 def head_mix(x: torch.Tensor, mix: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, d: int, dv: int,

@@ -58,8 +58,9 @@ def check(name, args):
             need(min(room(kc), room(vc)) >= val(pages) * nkv * page * d, "cache")
             need(int(ent.tensor[:tokens].max()) < bt.tensor.shape[0] and bt.tensor.shape[1] == width, "table")
             need(int(pos.tensor[:tokens].max()) // page < width, "a position beyond the table")
-    elif name == "pulse_attn_generic":
-        (q, qs, out, os_, _, _, _, _, pos, ent, bt, width, tokens, nq, _, d, page, _, _, _, gate, gs, _, _, _, _) = args
+    elif name == "pulse_attn_generic_ex":
+        (q, qs, out, os_, _, _, _, _, pos, ent, bt, width, tokens, nq, _, d, page, _, _, _, gate, gs, _, _, _, _, _, _,
+         _) = args
         tokens, nq, d = val(tokens), val(nq), val(d)
         need(room(q) >= (tokens - 1) * val(qs) + nq * d and room(out) >= (tokens - 1) * val(os_) + nq * d, "q / out")
         need(gate.tensor is None or room(gate) >= (tokens - 1) * val(gs) + nq, "gate")
@@ -102,7 +103,7 @@ def check(name, args):
         need(cout.tensor is None or room(cout) >= (m - 1) * val(ldcopy) + n, "copy")
         need(cscale.tensor is None or room(cscale) >= n, "copy scale")
     elif name == "pulse_add_rmsnorm":
-        (h, delta, _, parts, part_stride, rows, w, _, y, _, n_out, hidden, _, _, _, _) = args
+        (h, delta, _, parts, part_stride, rows, w, _, y, _, n_out, hidden, _, _, _, _, _) = args
         n_out, hidden = val(n_out), val(hidden)
         last = int(rows.tensor.max()) + 1 if rows.tensor is not None else n_out
         need(room(w) >= hidden and room(y) >= n_out * hidden and room(h) >= last * hidden, "w / y / h")
@@ -128,7 +129,7 @@ def check(name, args):
         ids, _, _, out, tokens, hidden, _, _, _, _ = args
         need(room(out) >= val(tokens) * val(hidden) and room(ids) >= val(tokens), "operands")
     elif name == "pulse_residual_add":
-        h, delta, _, parts, n, _ = args
+        h, delta, _, parts, n, _, _ = args
         need(room(h) >= val(n) and room(delta) >= val(parts) * val(n), "operands")
     elif name != "pulse_attn_plan":
         raise AssertionError(f"an entry point that nothing verifies: {name}")

@@ -575,9 +575,9 @@ def test_kernels_refuse_what_they_cannot_do(k):
         k.swiglu(torch.zeros(2, 4, dtype=torch.float16, device=DEV), torch.zeros(2, 2, dtype=torch.float16, device=DEV))
     with pytest.raises(KernelError, match="inner sizes"):
         k.gemm_f32(torch.zeros(2, 4, device=DEV), torch.zeros(3, 5, device=DEV), torch.zeros(2, 3, device=DEV))
-    kc, vc = _cache(2, 1, 4, 1024, torch.float32)
+    kc, vc = _cache(2, 1, 4, 4096, torch.float32)
     with pytest.raises(KernelError, match="head_dim"):
-        k.attn_generic(torch.zeros(1, 1024, device=DEV), torch.zeros(1, 1024, device=DEV), 1, 1, 1024, kc, vc,
+        k.attn_generic(torch.zeros(1, 4096, device=DEV), torch.zeros(1, 4096, device=DEV), 1, 1, 4096, kc, vc,
                        torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
                        torch.zeros(1, 1, dtype=torch.int32, device=DEV), 1.0)
 
