@@ -144,35 +144,32 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const bf16_t* __restrict
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int i = 0; i < 4; ++i) pb[4 * t + i] = static_cast<__bf16>(p[t][i]);
-        // O^T += V^T P^T, channel tile by channel tile
-        bool written[2][4];   // keys of the operand that have ever been stored
+        // O^T += V^T P^T, channel tile by channel tile.  Keys of the operand that have never been stored are cleared:
+        // one mask a 32-bit half of the lane's eight values, the same for every tile.
+        unsigned int keep_bits[4];
+        const bf16_t* vbase[2];
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) written[t][i] = page[t] >= 0 && jbase[t] + 4 * g + i <= pos_last;
+        for (int t = 0; t < 2; ++t) {
+            const int j = jbase[t] + 4 * g;
+            const bool there = page[t] >= 0;
+            keep_bits[2 * t] = (there && j <= pos_last ? 0x0000FFFFu : 0u) | (there && j + 1 <= pos_last ? 0xFFFF0000u : 0u);
+            keep_bits[2 * t + 1] = (there && j + 2 <= pos_last ? 0x0000FFFFu : 0u) | (there && j + 3 <= pos_last ? 0xFFFF0000u : 0u);
+            // (value head c's channel e lies (c * d + e) * page_size behind kv head 0's: with all values side by side the
+            // channel number is c * d + e itself)
+            vbase[t] = vcache + static_cast<int64_t>(there ? page[t] : 0) * a.nkv * d * a.page_size + off[t] + 4 * g
+                       + static_cast<int64_t>((a.all_values ? 0 : kvh * d) + chunk0 + r) * a.page_size;
+        }
+        const int tile_stride = 16 * a.page_size;
 #pragma unroll
         for (int c = 0; c < CHUNK_TILES; ++c) {
             if (c < tiles) {
                 acc[c] *= alpha;
-                const int ch = chunk0 + 16 * c + r;
-                const int vh = a.all_values ? ch / d : kvh;
-                const int e = a.all_values ? ch % d : ch;
-                u32x4 raw = {0u, 0u, 0u, 0u};
+                u32x4 raw;
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    if (page[t] >= 0) {
-                        const u32x2 two = *reinterpret_cast<const u32x2*>(
-                            vcache + ((static_cast<int64_t>(page[t]) * a.nkv + vh) * d + e) * a.page_size + off[t] + 4 * g);
-                        raw[2 * t] = two[0];
-                        raw[2 * t + 1] = two[1];
-                    }
-                }
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    if (!written[t][0]) raw[2 * t] &= 0xFFFF0000u;
-                    if (!written[t][1]) raw[2 * t] &= 0x0000FFFFu;
-                    if (!written[t][2]) raw[2 * t + 1] &= 0xFFFF0000u;
-                    if (!written[t][3]) raw[2 * t + 1] &= 0x0000FFFFu;
+                    const u32x2 two = *reinterpret_cast<const u32x2*>(vbase[t] + c * tile_stride);
+                    raw[2 * t] = two[0] & keep_bits[2 * t];
+                    raw[2 * t + 1] = two[1] & keep_bits[2 * t + 1];
                 }
                 acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, raw), pb, acc[c], 0, 0, 0);
             }

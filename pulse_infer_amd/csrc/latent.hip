@@ -9,6 +9,8 @@
 // pulse_latent_rows:   c and the turned key part into the pages; the queries' turned parts into their places.
 // pulse_latent_absorb: q_abs[t, h, :] = W_uk,h^T q_plain[t, h]        (float32 sums, one rounding)
 // pulse_latent_expand: y[t, h, :] = (W_uv,h o[t, h, :rank]) * sigmoid(gate[t, h, :])
+// pulse_heads_product: both of these products for bfloat16 weights on the matrix cores: y[t, h, m] = sum_k
+//                      w[h, m, k] x[t, h, k] (w_uk transposed once at load, w_uv as it is), 16 tokens a workgroup
 #include "common.h"
 
 #include <math.h>
@@ -120,6 +122,63 @@ __global__ void latent_expand_kernel(const TO* __restrict__ o, int64_t o_stride,
     }
 }
 
+
+// ------------------------------------------------------------------ a product a head, on the matrix cores
+typedef __attribute__((ext_vector_type(8))) __bf16 hp_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float hp_f32x4;
+
+template <typename T> __device__ __forceinline__ hp_bf16x8 load8(const T* p);
+template <> __device__ __forceinline__ hp_bf16x8 load8<bf16_t>(const bf16_t* p) { return *reinterpret_cast<const hp_bf16x8*>(p); }
+template <> __device__ __forceinline__ hp_bf16x8 load8<float>(const float* p) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    hp_bf16x8 out;
+    out[0] = static_cast<__bf16>(a.x); out[1] = static_cast<__bf16>(a.y); out[2] = static_cast<__bf16>(a.z); out[3] = static_cast<__bf16>(a.w);
+    out[4] = static_cast<__bf16>(b.x); out[5] = static_cast<__bf16>(b.y); out[6] = static_cast<__bf16>(b.z); out[7] = static_cast<__bf16>(b.w);
+    return out;
+}
+
+// A workgroup takes 16 tokens of one head; a wavefront a tile of 16 output channels at a time.  W rows are the matrix
+// cores' row operand (m = output channel), the tokens' rows of x the column operand, so a lane ends up with four
+// neighbouring channels of its token: one 8-byte store.
+template <typename TX>
+__global__ __launch_bounds__(256) void heads_product_kernel(const TX* __restrict__ x, int64_t x_stride, int x_head,
+                                                            const bf16_t* __restrict__ w, const bf16_t* __restrict__ gate,
+                                                            int64_t gate_stride, bf16_t* __restrict__ y, int64_t y_stride,
+                                                            int y_head, int tokens, int m_out, int k_in, float scale) {
+    const int t0 = blockIdx.x * 16, h = blockIdx.y;
+    const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
+    const int r = lane % 16, g = lane / 16;
+    const int tok = min(t0 + r, tokens - 1);
+    const TX* xrow = x + static_cast<int64_t>(tok) * x_stride + static_cast<int64_t>(h) * x_head;
+    const hp_bf16x8 zero = __builtin_bit_cast(hp_bf16x8, make_uint4(0u, 0u, 0u, 0u));
+    for (int m0 = wave * 16; m0 < m_out; m0 += 64) {
+        const int m = m0 + r;
+        const bf16_t* wrow = m < m_out ? w + (static_cast<int64_t>(h) * m_out + m) * k_in : nullptr;
+        hp_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int k0 = 0; k0 < k_in; k0 += 32) {
+            const int k = k0 + 8 * g;
+            const bool in = k < k_in;
+            const hp_bf16x8 wa = (in && wrow) ? *reinterpret_cast<const hp_bf16x8*>(wrow + k) : zero;
+            const hp_bf16x8 xb = in ? load8<TX>(xrow + k) : zero;
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xb, acc, 0, 0, 0);
+        }
+        // lane: token r, channels m0 + 4 g + i
+        if (t0 + r < tokens) {
+            const int c0 = m0 + 4 * g;
+            bf16_t* dst = y + static_cast<int64_t>(t0 + r) * y_stride + static_cast<int64_t>(h) * y_head + c0;
+            const bf16_t* gr = gate ? gate + static_cast<int64_t>(t0 + r) * gate_stride + static_cast<int64_t>(h) * m_out + c0 : nullptr;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (c0 + i < m_out) {
+                    float v = acc[i] * scale;
+                    if (gr) v *= 1.0f / (1.0f + expf(-bf16_to_f32(gr[i])));
+                    dst[i] = f32_to_bf16(v);
+                }
+            }
+        }
+    }
+}
+
 }  // namespace
 
 // x [tokens, x_stride]: the projection output; queries from column q0 (heads x (d + rot), the turned part last), the
@@ -187,5 +246,29 @@ extern "C" int pulse_latent_expand(const void* o, int64_t o_stride, int o_dtype,
                            static_cast<const TO*>(o), o_stride, stored, static_cast<const TW*>(w_uv),
                            static_cast<const TX*>(gate), gate_stride, static_cast<TX*>(y), y_stride, dv, rank, scale))));
     PULSE_LAUNCH_CHECK("latent_expand");
+    return 0;
+}
+
+// y[t, h * y_head + m] = scale * (sum_k w[h, m, k] * x[t, h * x_head + k]) * sigmoid(gate[t, h * m_out + m]) for bfloat16
+// w [heads, m_out, k_in] and y, x bfloat16 or float32 (rounded to bfloat16 as it is read); k_in a multiple of 8, rows
+// of x and w 16-byte aligned.  gate may be null.
+extern "C" int pulse_heads_product(const void* x, int64_t x_stride, int x_head, int x_dtype, const void* w, const void* gate,
+                                   int64_t gate_stride, void* y, int64_t y_stride, int y_head, int tokens, int heads,
+                                   int m_out, int k_in, float scale, hipStream_t stream) {
+    PULSE_REQUIRE(tokens >= 0 && heads > 0 && heads < 65536 && m_out > 0 && k_in > 0 && k_in % 8 == 0, "heads_product: bad sizes");
+    PULSE_REQUIRE(x && w && y && pulse_dtype_ok(x_dtype), "heads_product: bad arguments");
+    const int xb = x_dtype == PULSE_F32 ? 4 : 2;
+    PULSE_REQUIRE(x_head >= k_in && x_stride >= static_cast<int64_t>(heads - 1) * x_head + k_in &&
+                  y_head >= m_out && y_stride >= static_cast<int64_t>(heads - 1) * y_head + m_out &&
+                  (!gate || gate_stride >= static_cast<int64_t>(heads) * m_out), "heads_product: the rows are too short");
+    PULSE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && (x_stride * xb) % 16 == 0 && (static_cast<int64_t>(x_head) * xb) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(w) % 16 == 0, "heads_product: operands must be 16-byte aligned");
+    if (tokens == 0) return 0;
+    const dim3 grid((tokens + 15) / 16, heads);
+    PULSE_DISPATCH_DTYPE(x_dtype, TX,
+        hipLaunchKernelGGL(heads_product_kernel<TX>, grid, dim3(256), 0, stream, static_cast<const TX*>(x), x_stride, x_head,
+                           static_cast<const bf16_t*>(w), static_cast<const bf16_t*>(gate), gate_stride,
+                           static_cast<bf16_t*>(y), y_stride, y_head, tokens, m_out, k_in, scale));
+    PULSE_LAUNCH_CHECK("heads_product");
     return 0;
 }

@@ -714,6 +714,33 @@ def latent_expand(o: torch.Tensor, stored: int, w_uv: torch.Tensor, gate: Option
          _stream())
 
 
+def heads_product_takes(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, x_head: int) -> bool:
+    """Whether ``heads_product`` takes these operands (bfloat16 weights and results, aligned rows)."""
+    size = x.element_size()
+    return (w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and x.dtype in (torch.bfloat16, torch.float32)
+            and w.shape[2] % 8 == 0 and (x.stride(0) * size) % 16 == 0 and (x_head * size) % 16 == 0
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def heads_product(x: torch.Tensor, x_head: int, w: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor,
+                  out_head: int, scale: float = 1.0) -> None:
+    """out[t, h * out_head + m] = scale * (sum_k w[h, m, k] * x[t, h * x_head + k]) * sigmoid(gate[t, h * M + m]) on
+    the matrix cores: a product a head (w bfloat16 [heads, M, K]; x bfloat16 or float32; gate optional, of out's type)."""
+    _gpu("heads_product", x, w, gate, out)
+    tokens = x.shape[0]
+    heads, m_out, k_in = w.shape
+    _need(heads_product_takes(x, w, out, x_head) and w.is_contiguous(), "heads_product: bfloat16 weights [heads, M, K], aligned rows")
+    _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[1] >= (heads - 1) * x_head + k_in, "heads_product: x too narrow")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == tokens and out.shape[1] >= (heads - 1) * out_head + m_out,
+          "heads_product: out too narrow")
+    _need(gate is None or (gate.dtype == out.dtype and gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[0] == tokens
+                           and gate.shape[1] >= heads * m_out), "heads_product: the gate must be of out's type and width")
+    row = lambda t: t.stride(0) if tokens > 1 else t.shape[1]
+    call("pulse_heads_product", _ptr(x), _i64(row(x)), _i32(x_head), _i32(_tag(x, "heads_product")), _ptr(w), _ptr(gate),
+         _i64(row(gate) if gate is not None else 0), _ptr(out), _i64(row(out)), _i32(out_head), _i32(tokens), _i32(heads),
+         _i32(m_out), _i32(k_in), _f32(scale), _stream(), label=f"M={m_out} K={k_in}")
+
+
 def xielu(x: torch.Tensor, out: torch.Tensor, pq: torch.Tensor) -> None:
     """out = a z^2 + z / 2 for z > 0, else b (exp(z) - 1 - z) + z / 2, a = softplus(pq[0]), b = 1/2 + softplus(pq[1])."""
     _gpu("xielu", x, out, pq)

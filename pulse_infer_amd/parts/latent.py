@@ -104,6 +104,12 @@ class LatentAttention(PagedAttention):
         self.norm_weight = load.get(n["down_norm"])
         self.w_uk = load.get(n["up_k"])
         self.w_uv = load.get(n["up_v"])
+        # for the matrix cores: a head's rows side by side ([heads, out, in]); w_uk transposed once, so that both
+        # products walk their inner dimension along a row (a layout choice, not new maths)
+        self.w_uk_t = self.w_uv_h = None
+        if build.mode == "bfloat16" and self.w_uk.dtype == torch.bfloat16 and self.plain_dim % 8 == 0 and self.rank % 8 == 0:
+            self.w_uk_t = self.w_uk.view(self.nq, self.plain_dim, self.rank).transpose(1, 2).contiguous()
+            self.w_uv_h = self.w_uv.view(self.nq, self.v_dim, self.rank)
         self.sink = self._load_sink(load, n["sink"]) if params.get("sink", False) else None
         self._o_weight = load.get(n["o"])
         self._o = None
@@ -142,8 +148,11 @@ class LatentAttention(PagedAttention):
         kernels.latent_rows(y, 0, self.q_cols, q, self.norm_weight, tables.cos, tables.sin, tables.pairing, cache.keys,
                             cache.values, ctx.positions, ctx.token_entry, table, self.nq, self.plain_dim, self.rot_dim,
                             self.rank, self.d, self.eps, write=cache.writable)
-        kernels.latent_absorb(y, 0, self.plain_dim + self.rot_dim, self.w_uk, q, self.d, self.nq, self.plain_dim,
-                              self.rank)
+        q_head = self.plain_dim + self.rot_dim
+        if self.w_uk_t is not None and kernels.heads_product_takes(y, self.w_uk_t, q, q_head):
+            kernels.heads_product(y, q_head, self.w_uk_t, None, q, self.d)
+        else:
+            kernels.latent_absorb(y, 0, q_head, self.w_uk, q, self.d, self.nq, self.plain_dim, self.rank)
         # the weighted latent rows: from the matrix-core kernels of ``attention`` where they are compiled for rows this
         # wide (the activations' type), else in float32 from the matrix-core kernel for wide values or the generic one
         if self.uses_matrix_cores(q, cache):
@@ -163,7 +172,10 @@ class LatentAttention(PagedAttention):
             kernels.attn_generic(q, o, self.nq, 1, self.d, cache.keys, cache.values, ctx.positions, ctx.token_entry,
                                  table, self.scale, 0, sink=self.sink, softcap=self.score_cap)
         gate = y[:, self.gate_col0:self.gate_col0 + self.nq * self.v_dim] if self.gated else None
-        kernels.latent_expand(o, self.d, self.w_uv, gate, out, self.nq, self.v_dim, self.rank, self.out_scale)
+        if self.w_uv_h is not None and kernels.heads_product_takes(o, self.w_uv_h, out, self.d):
+            kernels.heads_product(o, self.d, self.w_uv_h, gate, out, self.v_dim, self.out_scale)
+        else:
+            kernels.latent_expand(o, self.d, self.w_uv, gate, out, self.nq, self.v_dim, self.rank, self.out_scale)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: PagedCacheView) -> torch.Tensor:
         if self._o is None:

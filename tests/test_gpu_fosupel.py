@@ -465,6 +465,17 @@ def test_latent_attention_from_its_projections_on(dtype, heads, d, dr, dv, rank,
         out = torch.full((len(positions), inner), float("nan"), dtype=dtype, device=DEV)
         kernels.latent_expand(o, D, w_uv, gate, out, heads, dv, rank)
         assert torch.allclose(out.cpu().to(F64), want, **tol(dtype)), (kind, float((out.cpu().to(F64) - want).abs().max()))
+        # the same two products a head on the matrix cores
+        w_uv_h = w_uv.view(heads, dv, rank)
+        if kernels.heads_product_takes(o, w_uv_h, out, D) and d % 8 == 0 and rank % 8 == 0:
+            again = torch.full((len(positions), inner), float("nan"), dtype=dtype, device=DEV)
+            kernels.heads_product(o, D, w_uv_h, gate, again, dv)
+            assert torch.allclose(again.cpu().to(F64), want, **tol(dtype)), (kind, "heads_product")
+            w_uk_t = w_uk.view(heads, d, rank).transpose(1, 2).contiguous()
+            q2 = q.clone()
+            q2.view(-1, heads, D)[:, :, :rank] = float("nan")
+            kernels.heads_product(step, d + dr, w_uk_t, None, q2, D)
+            assert torch.allclose(q2.float(), q.float(), atol=2e-2, rtol=2e-2)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
