@@ -2,9 +2,11 @@
 // side (a caller that mixes the heads' weights afterwards) or one wide latent row shared by all heads; with a window
 // that keeps a request's first tokens, and sinks.  bfloat16 operands, float32 everything else, float32 results.
 //
-// An item is 16 rows: `hp` query heads of one kv head for 16 / hp consecutive tokens of one request (a decoded token
-// is an item of its group's heads alone).  A workgroup takes an item and a chunk of up to 256 value channels; its four
-// wavefronts share the item's keys out in steps of 32 and meet in LDS at the end.  Per step and wavefront:
+// An item is R tiles of 16 rows: `hp` query heads of one kv head for 16 R / hp consecutive tokens of one request (a
+// decoded token is an item of its group's heads alone).  A workgroup takes an item and a chunk of 16 CT value channels;
+// its four wavefronts share the item's keys out in steps of 32 and meet in LDS at the end.  Every key and value
+// operand a wavefront fetches serves all R row tiles (R = 4, CT = 8 for prompt portions: the same accumulators as R =
+// 1, CT = 16 for decoded tokens, a quarter of the traffic a row).  Per step, row tile and wavefront:
 //
 //   S^T = K Q^T      two tiles of 16 keys x 16 rows (v_mfma_f32_16x16x32_bf16 over the head's channels): a lane then
 //                    holds, for ITS row (lane % 16), the scores of keys 4 (lane / 16) + i of both tiles;
@@ -28,8 +30,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
-constexpr int CHUNK_TILES = 16;             // channel tiles of 16 a workgroup accumulates
-constexpr int CHUNK = 16 * CHUNK_TILES;
+constexpr int MAX_TILES = 16;               // channel tiles of 16 a workgroup accumulates at most
 
 struct WideArgs {
     int nq, nkv, d;       // d: stored channels of a head (keys and values alike)
@@ -46,7 +47,8 @@ __device__ __forceinline__ bf16x8 zeros8() {
     return __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
 }
 
-__global__ __launch_bounds__(256) void attn_wide_kernel(const bf16_t* __restrict__ q, float* __restrict__ out,
+template <int R, int CT>
+__global__ __launch_bounds__(256, R == 1 ? 3 : 1) void attn_wide_kernel(const bf16_t* __restrict__ q, float* __restrict__ out,
                                                         const bf16_t* __restrict__ kcache,
                                                         const bf16_t* __restrict__ vcache,
                                                         const int* __restrict__ positions,
@@ -54,18 +56,27 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const bf16_t* __restrict
                                                         const int* __restrict__ block_table,
                                                         const int* __restrict__ items, const float* __restrict__ sink,
                                                         WideArgs a) {
-    __shared__ float red[3][CHUNK_TILES][PULSE_WAVE][4];
+    __shared__ float red[2][CT][PULSE_WAVE][4];
     __shared__ float ml[4][16][2];
     const int* it = items + 4 * blockIdx.x;
     const int t0 = it[0], nt = it[1], head0 = it[2], nh = it[3];
-    const int chunk0 = blockIdx.y * CHUNK;
-    const int tiles = min(CHUNK_TILES, (a.wv - chunk0) / 16);
+    const int chunk0 = blockIdx.y * (16 * CT);
+    const int tiles = min(CT, (a.wv - chunk0) / 16);
     const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
     const int r = lane % 16, g = lane / 16;
-    const int ti = r / a.hp, hi = r % a.hp;
-    const bool valid = ti < nt && hi < nh;
-    const int tok = t0 + (valid ? ti : 0), head = head0 + (valid ? hi : 0);
-    const int pos = positions[tok];
+    const int d = a.d;
+    bool valid[R];
+    int tok[R], head[R], pos[R];
+    const bf16_t* qrow[R];
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) {
+        const int row = 16 * rr + r, ti = row / a.hp, hi = row % a.hp;
+        valid[rr] = ti < nt && hi < nh;
+        tok[rr] = t0 + (valid[rr] ? ti : 0);
+        head[rr] = head0 + (valid[rr] ? hi : 0);
+        pos[rr] = positions[tok[rr]];
+        qrow[rr] = q + static_cast<int64_t>(tok[rr]) * a.q_stride + static_cast<int64_t>(head[rr]) * d;
+    }
     const int kvh = head0 / (a.nq / a.nkv);
     const int* bt = block_table + static_cast<int64_t>(token_entry[t0]) * a.bt_width;
     const int pos_first = positions[t0], pos_last = positions[t0 + nt - 1];
@@ -74,13 +85,16 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const bf16_t* __restrict
     const int nfirst = a.window > 0 ? min((a.keep_first + 15) & ~15, lo16) : 0;
     const int total = nfirst + pos_last + 1 - lo16;
     const int nsteps = (total + 31) / 32;
-    const int d = a.d;
-    const bf16_t* qrow = q + static_cast<int64_t>(tok) * a.q_stride + static_cast<int64_t>(head) * d;
 
-    float m_run = -INFINITY, l_run = 0.f;
-    f32x4 acc[CHUNK_TILES];
+    float m_run[R], l_run[R];
+    f32x4 acc[R][CT];
 #pragma unroll
-    for (int c = 0; c < CHUNK_TILES; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int rr = 0; rr < R; ++rr) {
+        m_run[rr] = -INFINITY;
+        l_run[rr] = 0.f;
+#pragma unroll
+        for (int c = 0; c < CT; ++c) acc[rr][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
 
     for (int step = wave; step < nsteps; step += 4) {
         int page[2], off[2], jbase[2];
@@ -94,8 +108,10 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const bf16_t* __restrict
             off[t] = jb % a.page_size;
             jbase[t] = jb;
         }
-        // S^T: keys x rows
-        f32x4 s[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+        // S^T: keys x rows, for every row tile from the same key operands
+        f32x4 s[R][2];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) s[rr][0] = s[rr][1] = f32x4{0.f, 0.f, 0.f, 0.f};
         const bf16_t* krow[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -104,46 +120,51 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const bf16_t* __restrict
         for (int e0 = 0; e0 < d; e0 += 32) {
             const int e = e0 + 8 * g;
             const bool in = e < d;
-            const bf16x8 qb = in ? *reinterpret_cast<const bf16x8*>(qrow + e) : zeros8();
+            bf16x8 ka[2];
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const bf16x8 ka = (in && krow[t]) ? *reinterpret_cast<const bf16x8*>(krow[t] + e) : zeros8();
-                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb, s[t], 0, 0, 0);
+            for (int t = 0; t < 2; ++t) ka[t] = (in && krow[t]) ? *reinterpret_cast<const bf16x8*>(krow[t] + e) : zeros8();
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr) {
+                const bf16x8 qb = in ? *reinterpret_cast<const bf16x8*>(qrow[rr] + e) : zeros8();
+#pragma unroll
+                for (int t = 0; t < 2; ++t) s[rr][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[t], qb, s[rr][t], 0, 0, 0);
             }
         }
-        // this row's scores of keys jbase[t] + 4 g + i
-        float v[2][4];
-        float mx = -INFINITY;
+        // every row's scores of keys jbase[t] + 4 g + i become its weights, in the order the P^T operand wants them
+        bf16x8 pb[R];
+        float alpha[R];
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int rr = 0; rr < R; ++rr) {
+            float v[2][4];
+            float mx = -INFINITY;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int j = jbase[t] + 4 * g + i;
-                const bool seen = valid && page[t] >= 0 && j <= pos && (a.window == 0 || pos - j < a.window || j < a.keep_first);
-                float x = s[t][i] * a.scale;
-                if (a.cap > 0.f) x = a.cap * tanhf(x / a.cap);
-                v[t][i] = seen ? x : -INFINITY;
-                mx = fmaxf(mx, v[t][i]);
-            }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, PULSE_WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, PULSE_WAVE));
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = (m_new == -INFINITY) ? 1.f : expf(m_run - m_new);
-        float p[2][4], sum = 0.f;
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+                for (int i = 0; i < 4; ++i) {
+                    const int j = jbase[t] + 4 * g + i;
+                    const bool seen = valid[rr] && page[t] >= 0 && j <= pos[rr] &&
+                                      (a.window == 0 || pos[rr] - j < a.window || j < a.keep_first);
+                    float x = s[rr][t][i] * a.scale;
+                    if (a.cap > 0.f) x = a.cap * tanhf(x / a.cap);
+                    v[t][i] = seen ? x : -INFINITY;
+                    mx = fmaxf(mx, v[t][i]);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, PULSE_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, PULSE_WAVE));
+            const float m_new = fmaxf(m_run[rr], mx);
+            alpha[rr] = (m_new == -INFINITY) ? 1.f : expf(m_run[rr] - m_new);
+            float sum = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                p[t][i] = (v[t][i] == -INFINITY) ? 0.f : expf(v[t][i] - m_new);
-                sum += p[t][i];
-            }
-        l_run = l_run * alpha + sum;
-        m_run = m_new;
-        bf16x8 pb;
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) pb[4 * t + i] = static_cast<__bf16>(p[t][i]);
+                for (int i = 0; i < 4; ++i) {
+                    const float p = (v[t][i] == -INFINITY) ? 0.f : expf(v[t][i] - m_new);
+                    sum += p;
+                    pb[rr][4 * t + i] = static_cast<__bf16>(p);
+                }
+            l_run[rr] = l_run[rr] * alpha[rr] + sum;
+            m_run[rr] = m_new;
+        }
         // O^T += V^T P^T, channel tile by channel tile.  Keys of the operand that have never been stored are cleared:
         // one mask a 32-bit half of the lane's eight values, the same for every tile.
         unsigned int keep_bits[4];
@@ -161,9 +182,8 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const bf16_t* __restrict
         }
         const int tile_stride = 16 * a.page_size;
 #pragma unroll
-        for (int c = 0; c < CHUNK_TILES; ++c) {
+        for (int c = 0; c < CT; ++c) {
             if (c < tiles) {
-                acc[c] *= alpha;
                 u32x4 raw;
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
@@ -171,54 +191,85 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const bf16_t* __restrict
                     raw[2 * t] = two[0] & keep_bits[2 * t];
                     raw[2 * t + 1] = two[1] & keep_bits[2 * t + 1];
                 }
-                acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, raw), pb, acc[c], 0, 0, 0);
+                const bf16x8 va = __builtin_bit_cast(bf16x8, raw);
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+                    acc[rr][c] *= alpha[rr];
+                    acc[rr][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[rr], acc[rr][c], 0, 0, 0);
+                }
             }
         }
     }
-    // a row's sum over the four lanes that share it; then the four wavefronts meet
-    l_run += __shfl_xor(l_run, 16, PULSE_WAVE);
-    l_run += __shfl_xor(l_run, 32, PULSE_WAVE);
-    if (g == 0) { ml[wave][r][0] = m_run; ml[wave][r][1] = l_run; }
-    __syncthreads();
-    float m_all = -INFINITY;
+    // row tile by row tile: a row's sum over the four lanes that share it; then the four wavefronts meet
 #pragma unroll
-    for (int w = 0; w < 4; ++w) m_all = fmaxf(m_all, ml[w][r][0]);
-    float l_all = 0.f;
+    for (int rr = 0; rr < R; ++rr) {
+        float l = l_run[rr];
+        l += __shfl_xor(l, 16, PULSE_WAVE);
+        l += __shfl_xor(l, 32, PULSE_WAVE);
+        __syncthreads();   // (the row tile before has been read)
+        if (g == 0) { ml[wave][r][0] = m_run[rr]; ml[wave][r][1] = l; }
+        __syncthreads();
+        float m_all = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) l_all += (ml[w][r][0] == -INFINITY) ? 0.f : ml[w][r][1] * expf(ml[w][r][0] - m_all);
-    const float mine = (m_run == -INFINITY) ? 0.f : expf(m_run - m_all);
+        for (int w = 0; w < 4; ++w) m_all = fmaxf(m_all, ml[w][r][0]);
+        float l_all = 0.f;
 #pragma unroll
-    for (int c = 0; c < CHUNK_TILES; ++c) {
-        if (c < tiles) {
-            acc[c] *= mine;
-            if (wave > 0) {
+        for (int w = 0; w < 4; ++w) l_all += (ml[w][r][0] == -INFINITY) ? 0.f : ml[w][r][1] * expf(ml[w][r][0] - m_all);
+        const float mine = (m_run[rr] == -INFINITY) ? 0.f : expf(m_run[rr] - m_all);
+        // the wavefronts' sums meet in two rounds (2 and 3 into 0 and 1, then 1 into 0): half the LDS of one round
 #pragma unroll
-                for (int i = 0; i < 4; ++i) red[wave - 1][c][lane][i] = acc[c][i];
+        for (int c = 0; c < CT; ++c) {
+            if (c < tiles) {
+                acc[rr][c] *= mine;
+                if (wave >= 2) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) red[wave - 2][c][lane][i] = acc[rr][c][i];
+                }
             }
         }
-    }
-    __syncthreads();
-    if (wave > 0) return;
-    // a sink is one more term of the softmax's denominator, exp(sink[h]), with no key and no value
-    float scale_out = 1.f;
-    if (sink) {
-        const float sk = sink[head];
-        if (m_all == -INFINITY) l_all = 1.f;
-        else if (sk > m_all) { scale_out = expf(m_all - sk); l_all = l_all * scale_out + 1.f; }
-        else l_all += expf(sk - m_all);
-    }
-    const float inv = l_all > 0.f ? scale_out / l_all : 0.f;
-    if (!valid) return;
-    float* orow = out + static_cast<int64_t>(tok) * a.o_stride + static_cast<int64_t>(head) * a.w + chunk0;
+        __syncthreads();
+        if (wave < 2) {
 #pragma unroll
-    for (int c = 0; c < CHUNK_TILES; ++c) {
-        if (c < tiles) {
-            f32x4 sum = acc[c];
+            for (int c = 0; c < CT; ++c) {
+                if (c < tiles) {
 #pragma unroll
-            for (int w = 0; w < 3; ++w)
+                    for (int i = 0; i < 4; ++i) acc[rr][c][i] += red[wave][c][lane][i];
+                }
+            }
+        }
+        __syncthreads();
+        if (wave == 1) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) sum[i] += red[w][c][lane][i];
-            *reinterpret_cast<f32x4*>(orow + 16 * c + 4 * g) = sum * inv;
+            for (int c = 0; c < CT; ++c) {
+                if (c < tiles) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) red[0][c][lane][i] = acc[rr][c][i];
+                }
+            }
+        }
+        __syncthreads();
+        if (wave == 0) {
+            // a sink is one more term of the softmax's denominator, exp(sink[h]), with no key and no value
+            float scale_out = 1.f;
+            if (sink) {
+                const float sk = sink[head[rr]];
+                if (m_all == -INFINITY) l_all = 1.f;
+                else if (sk > m_all) { scale_out = expf(m_all - sk); l_all = l_all * scale_out + 1.f; }
+                else l_all += expf(sk - m_all);
+            }
+            const float inv = l_all > 0.f ? scale_out / l_all : 0.f;
+            if (valid[rr]) {
+                float* orow = out + static_cast<int64_t>(tok[rr]) * a.o_stride + static_cast<int64_t>(head[rr]) * a.w + chunk0;
+#pragma unroll
+                for (int c = 0; c < CT; ++c) {
+                    if (c < tiles) {
+                        f32x4 sum = acc[rr][c];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) sum[i] += red[0][c][lane][i];
+                        *reinterpret_cast<f32x4*>(orow + 16 * c + 4 * g) = sum * inv;
+                    }
+                }
+            }
         }
     }
 }
@@ -227,18 +278,19 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const bf16_t* __restrict
 
 // q [tokens, q_stride] bfloat16: head h's query at h * d.  out float32 [tokens, o_stride]: head h's result at h * w,
 // w = nkv * d with all_values (value head c at c * d) else d; channels 0 .. wv - 1 of it are written.  items int32
-// [n_items, 4]: first token, tokens, first head, heads; row r of an item is token r / hp, head r % hp.  kcache
+// [n_items, 4]: first token, tokens, first head, heads; row r (of 16 row_tiles, row_tiles 1 or 4) of an item is token
+// r / hp, head r % hp.  kcache
 // [pages, nkv, page, d], vcache [pages, nkv, d, page] bfloat16, page_size a multiple of 16, d a multiple of 16.
 extern "C" int pulse_attn_wide(const void* q, int64_t q_stride, float* out, int64_t o_stride, const void* kcache,
                                const void* vcache, const int* positions, const int* token_entry, const int* block_table,
-                               int bt_width, const int* items, int n_items, int hp, int nq, int nkv, int d, int wv,
+                               int bt_width, const int* items, int n_items, int hp, int row_tiles, int nq, int nkv, int d, int wv,
                                int all_values, int page_size, int num_pages, float scale, int window, int keep_first,
                                const float* sink, float softcap, hipStream_t stream) {
     PULSE_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0 && d > 0 && d % 16 == 0, "attn_wide: bad head sizes");
     PULSE_REQUIRE(page_size > 0 && page_size % 16 == 0 && num_pages > 0 && bt_width > 0, "attn_wide: pages must hold a multiple of 16 keys");
     const int w = all_values ? nkv * d : d;
     PULSE_REQUIRE(wv > 0 && wv % 16 == 0 && wv <= w, "attn_wide: %d of %d value channels", wv, w);
-    PULSE_REQUIRE(hp >= 1 && hp <= 16 && n_items >= 0, "attn_wide: bad items");
+    PULSE_REQUIRE(hp >= 1 && hp <= 16 && n_items >= 0 && (row_tiles == 1 || row_tiles == 4), "attn_wide: bad items");
     PULSE_REQUIRE(window >= 0 && keep_first >= 0 && softcap >= 0.f, "attn_wide: bad window, kept keys or score cap");
     PULSE_REQUIRE(q_stride >= static_cast<int64_t>(nq) * d && o_stride >= static_cast<int64_t>(nq) * w && o_stride % 4 == 0 &&
                   q_stride % 8 == 0, "attn_wide: row strides too small or unaligned");
@@ -251,10 +303,17 @@ extern "C" int pulse_attn_wide(const void* q, int64_t q_stride, float* out, int6
     a.nq = nq; a.nkv = nkv; a.d = d; a.w = w; a.wv = wv; a.all_values = all_values ? 1 : 0; a.hp = hp;
     a.q_stride = q_stride; a.o_stride = o_stride; a.page_size = page_size; a.num_pages = num_pages; a.bt_width = bt_width;
     a.scale = scale; a.cap = softcap; a.window = window; a.keep_first = window > 0 ? keep_first : 0;
-    const dim3 grid(n_items, (wv + CHUNK - 1) / CHUNK);
-    hipLaunchKernelGGL(attn_wide_kernel, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(q), out,
-                       static_cast<const bf16_t*>(kcache), static_cast<const bf16_t*>(vcache), positions, token_entry,
-                       block_table, items, sink, a);
+    if (row_tiles == 4) {
+        const dim3 grid(n_items, (wv + 127) / 128);
+        hipLaunchKernelGGL((attn_wide_kernel<4, 8>), grid, dim3(256), 0, stream, static_cast<const bf16_t*>(q), out,
+                           static_cast<const bf16_t*>(kcache), static_cast<const bf16_t*>(vcache), positions, token_entry,
+                           block_table, items, sink, a);
+    } else {
+        const dim3 grid(n_items, (wv + 255) / 256);
+        hipLaunchKernelGGL((attn_wide_kernel<1, MAX_TILES>), grid, dim3(256), 0, stream, static_cast<const bf16_t*>(q), out,
+                           static_cast<const bf16_t*>(kcache), static_cast<const bf16_t*>(vcache), positions, token_entry,
+                           block_table, items, sink, a);
+    }
     PULSE_LAUNCH_CHECK("attn_wide");
     return 0;
 }

@@ -541,13 +541,25 @@ def attn_wide_takes(q: torch.Tensor, kcache: torch.Tensor, d: int) -> bool:
             and kcache.shape[2] % 16 == 0 and d % 16 == 0)
 
 
-def attn_wide_items(entries, nq: int, nkv: int):
-    """The work list of ``attn_wide`` for a step's entries (anything with ``first_row`` and ``count``): items of 16
-    rows, ``hp`` heads of one kv head for 16 // hp consecutive tokens of one entry.  Returns (flat list of
-    quadruples first token, tokens, first head, heads; hp)."""
+WIDE_ROW_TILES = (1, 4)     # row tiles of 16 an item of ``attn_wide`` may have
+
+
+def attn_wide_row_tiles(tokens: int) -> int:
+    """Row tiles an item gets in a step of ``tokens`` tokens.  Always 1: items of 4 row tiles (every key and value
+    fetched serves four times the rows, 128 value channels a workgroup) need all the registers a wavefront can have, so
+    a compute unit holds a wavefront a SIMD, and a prompt of 2,048 tokens took 1.5 times as long with them (window
+    attention over 8 kv heads' values 6.7 ms against 4.5 for three layers, a latent row of 576 channels 3.2 against
+    2.2): what bounds this kernel is the trips to memory that a wavefront waits for, not the bytes."""
+    return WIDE_ROW_TILES[0]
+
+
+def attn_wide_items(entries, nq: int, nkv: int, row_tiles: int = 1):
+    """The work list of ``attn_wide`` for a step's entries (anything with ``first_row`` and ``count``): items of
+    16 row_tiles rows, ``hp`` heads of one kv head for 16 row_tiles // hp consecutive tokens of one entry.  Returns (flat
+    list of quadruples first token, tokens, first head, heads; hp)."""
     group = nq // nkv
     hp = min(group, 16)
-    tp = 16 // hp
+    tp = 16 * row_tiles // hp
     flat = []
     for e in entries:
         for t in range(0, e.count, tp):
@@ -561,7 +573,7 @@ def attn_wide_items(entries, nq: int, nkv: int):
 def attn_wide(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, wv: int, all_values: bool,
               kcache: torch.Tensor, vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor,
               block_table: torch.Tensor, items: torch.Tensor, hp: int, scale: float, window: int = 0,
-              keep_first: int = 0, sink: Optional[torch.Tensor] = None, softcap: float = 0.0) -> None:
+              keep_first: int = 0, sink: Optional[torch.Tensor] = None, softcap: float = 0.0, row_tiles: int = 1) -> None:
     """Paged attention on the matrix cores for heads that gather wide values: with ``all_values`` every query head's
     weights on the values of all kv heads (out float32 [T, nq * nkv * d], as ``attn_generic`` leaves it), else on its
     own kv head's (out float32 [T, nq * d]); of a head's channels the first ``wv`` (a multiple of 16) are written.
@@ -569,6 +581,7 @@ def attn_wide(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, wv:
     _gpu("attn_wide", q, out, kcache, vcache, positions, token_entry, block_table, items, sink)
     tokens = q.shape[0]
     _need(attn_wide_takes(q, kcache, d), "attn_wide: bfloat16 operands, pages of a multiple of 16 keys, d % 16 == 0")
+    _need(row_tiles in WIDE_ROW_TILES, f"attn_wide: items of {WIDE_ROW_TILES} row tiles, not {row_tiles}")
     width = nq * d * (nkv if all_values else 1)
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * d, "attn_wide: q too narrow")
     _need(out.dtype == torch.float32 and out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == tokens
@@ -583,9 +596,9 @@ def attn_wide(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, wv:
         _need(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == nq, f"attn_wide: the sinks must be float32 [{nq}]")
     call("pulse_attn_wide", _ptr(q), _i64(q.stride(0) if tokens > 1 else q.shape[1]), _ptr(out),
          _i64(out.stride(0) if tokens > 1 else out.shape[1]), _ptr(kcache), _ptr(vcache), _ptr(positions), _ptr(token_entry),
-         _ptr(block_table), _i32(block_table.shape[1]), _ptr(items), _i32(items.numel() // 4), _i32(hp), _i32(nq), _i32(nkv),
-         _i32(d), _i32(wv), _i32(1 if all_values else 0), _i32(page_size), _i32(pages), _f32(scale), _i32(window),
-         _i32(keep_first), _ptr(sink), _f32(softcap), _stream(), label=f"d={d} values={wv}")
+         _ptr(block_table), _i32(block_table.shape[1]), _ptr(items), _i32(items.numel() // 4), _i32(hp), _i32(row_tiles),
+         _i32(nq), _i32(nkv), _i32(d), _i32(wv), _i32(1 if all_values else 0), _i32(page_size), _i32(pages), _f32(scale), _i32(window),
+         _i32(keep_first), _ptr(sink), _f32(softcap), _stream(), label=f"d={d} values={wv} tiles={row_tiles}")
 
 
 def head_mix(x: torch.Tensor, mix: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, d: int, dv: int,

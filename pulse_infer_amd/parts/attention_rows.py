@@ -203,10 +203,10 @@ class RowPreparedAttention(PagedAttention):
         width = self.nq * self.d * (self.nkv if self.talks else 1)
         each = ws.buffer("attention_rows.each", tokens, width, torch.float32)
         if wide:
-            items, hp = self._wide_items(ctx)
+            items, hp, row_tiles = self._wide_items(ctx)
             kernels.attn_wide(q, each, self.nq, self.nkv, self.d, self.nkv * self.d if self.talks else self.d, self.talks,
                               cache.keys, cache.values, ctx.positions, ctx.token_entry, table, items, hp, self.scale,
-                              window, self.keep_first, self.sink, self.score_cap)
+                              window, self.keep_first, self.sink, self.score_cap, row_tiles)
         else:
             kernels.attn_generic(q, each, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
                                  ctx.token_entry, table, self.scale, window, sink=self.sink, softcap=self.score_cap,
@@ -221,8 +221,9 @@ class RowPreparedAttention(PagedAttention):
         head counts shares it)."""
         key = f"static:attention_rows.wide_items:{self.nq}:{self.nkv}"
         if key not in ctx.extras:
-            flat, hp = kernels.attn_wide_items(ctx.entries, self.nq, self.nkv)
-            ctx.extras[key] = (ctx.to_device(flat), hp)
+            row_tiles = kernels.attn_wide_row_tiles(ctx.num_tokens)
+            flat, hp = kernels.attn_wide_items(ctx.entries, self.nq, self.nkv, row_tiles)
+            ctx.extras[key] = (ctx.to_device(flat), hp, row_tiles)
         return ctx.extras[key]
 
     def _identity(self, device) -> torch.Tensor:

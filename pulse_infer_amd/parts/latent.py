@@ -162,11 +162,13 @@ class LatentAttention(PagedAttention):
             o = ws.buffer("latent.rows", tokens, self.nq * self.d, torch.float32)
             key = f"static:latent.wide_items:{self.nq}"
             if key not in ctx.extras:
-                flat, hp = kernels.attn_wide_items(ctx.entries, self.nq, 1)
-                ctx.extras[key] = (ctx.to_device(flat), hp)
-            items, hp = ctx.extras[key]
+                row_tiles = kernels.attn_wide_row_tiles(ctx.num_tokens)
+                flat, hp = kernels.attn_wide_items(ctx.entries, self.nq, 1, row_tiles)
+                ctx.extras[key] = (ctx.to_device(flat), hp, row_tiles)
+            items, hp, row_tiles = ctx.extras[key]
             kernels.attn_wide(q, o, self.nq, 1, self.d, (self.rank + 15) // 16 * 16, False, cache.keys, cache.values,
-                              ctx.positions, ctx.token_entry, table, items, hp, self.scale, 0, 0, self.sink, self.score_cap)
+                              ctx.positions, ctx.token_entry, table, items, hp, self.scale, 0, 0, self.sink, self.score_cap,
+                              row_tiles)
         else:
             o = ws.buffer("latent.rows", tokens, self.nq * self.d, torch.float32)
             kernels.attn_generic(q, o, self.nq, 1, self.d, cache.keys, cache.values, ctx.positions, ctx.token_entry,

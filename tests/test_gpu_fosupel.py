@@ -288,17 +288,18 @@ def test_kept_first_tokens_window_sinks_and_mixed_heads(case, dtype, needle):
         def __init__(self, first_row, count):
             self.first_row, self.count = first_row, count
     step_entries = [E(0, portion)] + [E(portion + i, 1) for i in range(len(lens) - 1)]
-    paths = ["generic"] + (["wide"] if kernels.attn_wide_takes(q, kc, d) else [])
+    paths = ["generic"] + (["wide", "wide4"] if kernels.attn_wide_takes(q, kc, d) else [])
     assert dtype != torch.bfloat16 or bs % 16 or d % 16 or "wide" in paths
     for path in paths:
+        row_tiles = 4 if path == "wide4" else 1
         each = torch.full((len(positions), nq * nkv * d), float("nan"), dtype=torch.float32, device=DEV)
         if path == "generic":
             kernels.attn_generic(q, each, nq, nkv, d, kc, vc, ints(positions), ints(entry), table.to(DEV), scale, window,
                                  sink=sink.to(DEV), keep_first=keep, all_values=True)
         else:
-            flat, hp = kernels.attn_wide_items(step_entries, nq, nkv)
+            flat, hp = kernels.attn_wide_items(step_entries, nq, nkv, row_tiles)
             kernels.attn_wide(q, each, nq, nkv, d, nkv * d, True, kc, vc, ints(positions), ints(entry), table.to(DEV),
-                              ints(flat), hp, scale, window, keep, sink.to(DEV))
+                              ints(flat), hp, scale, window, keep, sink.to(DEV), row_tiles=row_tiles)
         out = torch.full((len(positions), nq * d), float("nan"), dtype=dtype, device=DEV)
         kernels.head_mix(each, mix, out, nq, nkv, d, dv, d, 0.8)
         got = out.cpu().to(F64).view(-1, nq, d)
@@ -313,10 +314,10 @@ def test_kept_first_tokens_window_sinks_and_mixed_heads(case, dtype, needle):
             assert torch.allclose(got[row:row + rows, :, :dv], want, **tol(dtype)), \
                 (path, r, float((got[row:row + rows, :, :dv] - want).abs().max()))
             row += rows
-        if path == "wide":   # a head's own values alone, as the part asks for them without mixed heads
+        if path != "generic":   # a head's own values alone, as the part asks for them without mixed heads
             own = torch.full((len(positions), nq * d), float("nan"), dtype=torch.float32, device=DEV)
             kernels.attn_wide(q, own, nq, nkv, d, d, False, kc, vc, ints(positions), ints(entry), table.to(DEV),
-                              ints(flat), hp, scale, window, keep, sink.to(DEV))
+                              ints(flat), hp, scale, window, keep, sink.to(DEV), row_tiles=row_tiles)
             got, row = own.cpu().to(F64).view(-1, nq, d), 0
             for r, n in enumerate(lens):
                 rows = portion if r == 0 else 1
@@ -446,16 +447,18 @@ def test_latent_attention_from_its_projections_on(dtype, heads, d, dr, dv, rank,
         def __init__(self, first_row, count):
             self.first_row, self.count = first_row, count
     paths = [torch.float32] + ([dtype] if M.supported(D, bs, dtype, dtype) else [])
-    paths += ["wide"] if kernels.attn_wide_takes(q, kc, D) else []
+    paths += ["wide", "wide4"] if kernels.attn_wide_takes(q, kc, D) else []
     for kind in paths:
-        o = torch.full((len(positions), heads * D), float("nan"), dtype=torch.float32 if kind == "wide" else kind, device=DEV)
+        o = torch.full((len(positions), heads * D), float("nan"), dtype=torch.float32 if kind in ("wide", "wide4") else kind, device=DEV)
         if kind == torch.float32:
             kernels.attn_generic(q, o, heads, 1, D, kc, vc, ints(positions), ints(entry), table.to(DEV), scale, 0,
                                  sink=sink.to(DEV))
-        elif kind == "wide":
-            flat, hp = kernels.attn_wide_items([E(0, portion)] + [E(portion + i, 1) for i in range(len(lens) - 1)], heads, 1)
+        elif kind in ("wide", "wide4"):
+            row_tiles = 4 if kind == "wide4" else 1
+            flat, hp = kernels.attn_wide_items([E(0, portion)] + [E(portion + i, 1) for i in range(len(lens) - 1)], heads, 1,
+                                               row_tiles)
             kernels.attn_wide(q, o, heads, 1, D, (rank + 15) // 16 * 16, False, kc, vc, ints(positions), ints(entry),
-                              table.to(DEV), ints(flat), hp, scale, 0, 0, sink.to(DEV))
+                              table.to(DEV), ints(flat), hp, scale, 0, 0, sink.to(DEV), row_tiles=row_tiles)
         else:
             numbered = list(enumerate([E(0, portion)] + [E(portion + i, 1) for i in range(len(lens) - 1)]))
             items = ints(M.build_items(numbered, M.tokens_per_item(heads)))
