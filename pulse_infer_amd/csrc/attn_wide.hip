@@ -41,6 +41,9 @@ struct WideArgs {
     int page_size, num_pages, bt_width;
     float scale, cap;
     int window, keep_first;
+    int n_splits;         // > 1: the keys' steps are shared out over gridDim.z workgroups, whose sums go to `part`
+    float* part;          // [tokens, nq, n_splits, w] sums not yet divided
+    float* part_ml;       // [tokens, nq, n_splits, 2] maximum and sum of weights
 };
 
 __device__ __forceinline__ bf16x8 zeros8() {
@@ -96,7 +99,9 @@ __global__ __launch_bounds__(256, R == 1 ? 3 : 1) void attn_wide_kernel(const bf
         for (int c = 0; c < CT; ++c) acc[rr][c] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    for (int step = wave; step < nsteps; step += 4) {
+    const int per_split = (nsteps + a.n_splits - 1) / a.n_splits;
+    const int step0 = static_cast<int>(blockIdx.z) * per_split, step1 = min(nsteps, step0 + per_split);
+    for (int step = step0 + wave; step < step1; step += 4) {
         int page[2], off[2], jbase[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -248,7 +253,23 @@ __global__ __launch_bounds__(256, R == 1 ? 3 : 1) void attn_wide_kernel(const bf
             }
         }
         __syncthreads();
-        if (wave == 0) {
+        if (wave == 0 && a.n_splits > 1) {
+            // one of several workgroups over these keys: the sums as they are, for the merge
+            if (valid[rr]) {
+                const int64_t at = (static_cast<int64_t>(tok[rr]) * a.nq + head[rr]) * a.n_splits + blockIdx.z;
+                if (blockIdx.y == 0 && g == 0) { a.part_ml[2 * at] = m_all; a.part_ml[2 * at + 1] = l_all; }
+                float* prow = a.part + at * a.w + chunk0;
+#pragma unroll
+                for (int c = 0; c < CT; ++c) {
+                    if (c < tiles) {
+                        f32x4 sum = acc[rr][c];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) sum[i] += red[0][c][lane][i];
+                        *reinterpret_cast<f32x4*>(prow + 16 * c + 4 * g) = sum;
+                    }
+                }
+            }
+        } else if (wave == 0) {
             // a sink is one more term of the softmax's denominator, exp(sink[h]), with no key and no value
             float scale_out = 1.f;
             if (sink) {
@@ -274,24 +295,61 @@ __global__ __launch_bounds__(256, R == 1 ? 3 : 1) void attn_wide_kernel(const bf
     }
 }
 
+// The sums of the workgroups that shared a row's keys, brought together: a workgroup a (token, head).
+__global__ void attn_wide_merge_kernel(const float* __restrict__ part, const float* __restrict__ part_ml,
+                                       float* __restrict__ out, int64_t o_stride, const float* __restrict__ sink, int nq,
+                                       int w, int wv, int n_splits) {
+    const int tok = blockIdx.x, head = blockIdx.y;
+    const int64_t at = (static_cast<int64_t>(tok) * nq + head) * n_splits;
+    float m_all = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) m_all = fmaxf(m_all, part_ml[2 * (at + s)]);
+    float l_all = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float m = part_ml[2 * (at + s)];
+        l_all += (m == -INFINITY) ? 0.f : part_ml[2 * (at + s) + 1] * expf(m - m_all);
+    }
+    float scale_out = 1.f;
+    if (sink) {
+        const float sk = sink[head];
+        if (m_all == -INFINITY) l_all = 1.f;
+        else if (sk > m_all) { scale_out = expf(m_all - sk); l_all = l_all * scale_out + 1.f; }
+        else l_all += expf(sk - m_all);
+    }
+    const float inv = l_all > 0.f ? scale_out / l_all : 0.f;
+    float* orow = out + static_cast<int64_t>(tok) * o_stride + static_cast<int64_t>(head) * w;
+    for (int ch = threadIdx.x; ch < wv; ch += blockDim.x) {
+        float sum = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float m = part_ml[2 * (at + s)];
+            if (m != -INFINITY) sum = fmaf(part[(at + s) * w + ch], expf(m - m_all), sum);
+        }
+        orow[ch] = sum * inv;
+    }
+}
+
 }  // namespace
 
 // q [tokens, q_stride] bfloat16: head h's query at h * d.  out float32 [tokens, o_stride]: head h's result at h * w,
 // w = nkv * d with all_values (value head c at c * d) else d; channels 0 .. wv - 1 of it are written.  items int32
 // [n_items, 4]: first token, tokens, first head, heads; row r (of 16 row_tiles, row_tiles 1 or 4) of an item is token
-// r / hp, head r % hp.  kcache
+// r / hp, head r % hp; the items must cover every (token, head) of the `tokens` tokens.  n_splits > 1: the keys of
+// every item are shared out over that many workgroups, whose sums (part float32 [tokens, nq, n_splits, w], part_ml
+// [tokens, nq, n_splits, 2]) a second kernel brings together.  kcache
 // [pages, nkv, page, d], vcache [pages, nkv, d, page] bfloat16, page_size a multiple of 16, d a multiple of 16.
 extern "C" int pulse_attn_wide(const void* q, int64_t q_stride, float* out, int64_t o_stride, const void* kcache,
                                const void* vcache, const int* positions, const int* token_entry, const int* block_table,
                                int bt_width, const int* items, int n_items, int hp, int row_tiles, int nq, int nkv, int d, int wv,
                                int all_values, int page_size, int num_pages, float scale, int window, int keep_first,
-                               const float* sink, float softcap, hipStream_t stream) {
+                               const float* sink, float softcap, int n_splits, float* part, float* part_ml, int tokens,
+                               hipStream_t stream) {
     PULSE_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0 && d > 0 && d % 16 == 0, "attn_wide: bad head sizes");
     PULSE_REQUIRE(page_size > 0 && page_size % 16 == 0 && num_pages > 0 && bt_width > 0, "attn_wide: pages must hold a multiple of 16 keys");
     const int w = all_values ? nkv * d : d;
     PULSE_REQUIRE(wv > 0 && wv % 16 == 0 && wv <= w, "attn_wide: %d of %d value channels", wv, w);
     PULSE_REQUIRE(hp >= 1 && hp <= 16 && n_items >= 0 && (row_tiles == 1 || row_tiles == 4), "attn_wide: bad items");
     PULSE_REQUIRE(window >= 0 && keep_first >= 0 && softcap >= 0.f, "attn_wide: bad window, kept keys or score cap");
+    PULSE_REQUIRE(n_splits >= 1 && n_splits <= 64 && tokens >= 0 && (n_splits == 1 || (part && part_ml)),
+                  "attn_wide: %d splits need their scratch", n_splits);
     PULSE_REQUIRE(q_stride >= static_cast<int64_t>(nq) * d && o_stride >= static_cast<int64_t>(nq) * w && o_stride % 4 == 0 &&
                   q_stride % 8 == 0, "attn_wide: row strides too small or unaligned");
     PULSE_REQUIRE(q && out && kcache && vcache && positions && token_entry && block_table && items, "attn_wide: null pointer");
@@ -303,17 +361,24 @@ extern "C" int pulse_attn_wide(const void* q, int64_t q_stride, float* out, int6
     a.nq = nq; a.nkv = nkv; a.d = d; a.w = w; a.wv = wv; a.all_values = all_values ? 1 : 0; a.hp = hp;
     a.q_stride = q_stride; a.o_stride = o_stride; a.page_size = page_size; a.num_pages = num_pages; a.bt_width = bt_width;
     a.scale = scale; a.cap = softcap; a.window = window; a.keep_first = window > 0 ? keep_first : 0;
+    a.n_splits = n_splits; a.part = part; a.part_ml = part_ml;
     if (row_tiles == 4) {
-        const dim3 grid(n_items, (wv + 127) / 128);
+        const dim3 grid(n_items, (wv + 127) / 128, n_splits);
         hipLaunchKernelGGL((attn_wide_kernel<4, 8>), grid, dim3(256), 0, stream, static_cast<const bf16_t*>(q), out,
                            static_cast<const bf16_t*>(kcache), static_cast<const bf16_t*>(vcache), positions, token_entry,
                            block_table, items, sink, a);
     } else {
-        const dim3 grid(n_items, (wv + 255) / 256);
+        const dim3 grid(n_items, (wv + 255) / 256, n_splits);
         hipLaunchKernelGGL((attn_wide_kernel<1, MAX_TILES>), grid, dim3(256), 0, stream, static_cast<const bf16_t*>(q), out,
                            static_cast<const bf16_t*>(kcache), static_cast<const bf16_t*>(vcache), positions, token_entry,
                            block_table, items, sink, a);
     }
     PULSE_LAUNCH_CHECK("attn_wide");
+    if (n_splits > 1 && tokens > 0) {
+        // (every (token, head) of the step has been written by the items: the work list covers them all)
+        hipLaunchKernelGGL(attn_wide_merge_kernel, dim3(tokens, nq), dim3(256), 0, stream, part, part_ml, out, o_stride, sink,
+                           nq, w, wv, n_splits);
+        PULSE_LAUNCH_CHECK("attn_wide_merge");
+    }
     return 0;
 }

@@ -573,7 +573,8 @@ def attn_wide_items(entries, nq: int, nkv: int, row_tiles: int = 1):
 def attn_wide(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, wv: int, all_values: bool,
               kcache: torch.Tensor, vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor,
               block_table: torch.Tensor, items: torch.Tensor, hp: int, scale: float, window: int = 0,
-              keep_first: int = 0, sink: Optional[torch.Tensor] = None, softcap: float = 0.0, row_tiles: int = 1) -> None:
+              keep_first: int = 0, sink: Optional[torch.Tensor] = None, softcap: float = 0.0, row_tiles: int = 1,
+              n_splits: int = 1, part: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None) -> None:
     """Paged attention on the matrix cores for heads that gather wide values: with ``all_values`` every query head's
     weights on the values of all kv heads (out float32 [T, nq * nkv * d], as ``attn_generic`` leaves it), else on its
     own kv head's (out float32 [T, nq * d]); of a head's channels the first ``wv`` (a multiple of 16) are written.
@@ -582,6 +583,13 @@ def attn_wide(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, wv:
     tokens = q.shape[0]
     _need(attn_wide_takes(q, kcache, d), "attn_wide: bfloat16 operands, pages of a multiple of 16 keys, d % 16 == 0")
     _need(row_tiles in WIDE_ROW_TILES, f"attn_wide: items of {WIDE_ROW_TILES} row tiles, not {row_tiles}")
+    if n_splits > 1:
+        _gpu("attn_wide", part, part_ml)
+        head_width = d * (nkv if all_values else 1)
+        _need(part is not None and part.dtype == torch.float32 and part.is_contiguous()
+              and part.numel() >= tokens * nq * n_splits * head_width, "attn_wide: the splits' scratch is too small")
+        _need(part_ml is not None and part_ml.dtype == torch.float32 and part_ml.is_contiguous()
+              and part_ml.numel() >= tokens * nq * n_splits * 2, "attn_wide: the splits' scratch is too small")
     width = nq * d * (nkv if all_values else 1)
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * d, "attn_wide: q too narrow")
     _need(out.dtype == torch.float32 and out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == tokens
@@ -598,7 +606,18 @@ def attn_wide(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, wv:
          _i64(out.stride(0) if tokens > 1 else out.shape[1]), _ptr(kcache), _ptr(vcache), _ptr(positions), _ptr(token_entry),
          _ptr(block_table), _i32(block_table.shape[1]), _ptr(items), _i32(items.numel() // 4), _i32(hp), _i32(row_tiles),
          _i32(nq), _i32(nkv), _i32(d), _i32(wv), _i32(1 if all_values else 0), _i32(page_size), _i32(pages), _f32(scale), _i32(window),
-         _i32(keep_first), _ptr(sink), _f32(softcap), _stream(), label=f"d={d} values={wv} tiles={row_tiles}")
+         _i32(keep_first), _ptr(sink), _f32(softcap), _i32(n_splits), _ptr(part if n_splits > 1 else None),
+         _ptr(part_ml if n_splits > 1 else None), _i32(tokens), _stream(),
+         label=f"d={d} values={wv} tiles={row_tiles} splits={n_splits}")
+
+
+def attn_wide_splits(n_items: int, chunks: int, keys: int) -> int:
+    """Over how many workgroups ``attn_wide`` shares an item's keys out: enough that the launch has about two
+    workgroups a compute unit, every one with at least four steps of 32 keys."""
+    from .device import compute_units
+    base = max(1, n_items * chunks)
+    want = (2 * compute_units() + base - 1) // base
+    return max(1, min(want, 16, keys // 128))
 
 
 def head_mix(x: torch.Tensor, mix: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, d: int, dv: int,

@@ -204,9 +204,16 @@ class RowPreparedAttention(PagedAttention):
         each = ws.buffer("attention_rows.each", tokens, width, torch.float32)
         if wide:
             items, hp, row_tiles = self._wide_items(ctx)
-            kernels.attn_wide(q, each, self.nq, self.nkv, self.d, self.nkv * self.d if self.talks else self.d, self.talks,
-                              cache.keys, cache.values, ctx.positions, ctx.token_entry, table, items, hp, self.scale,
-                              window, self.keep_first, self.sink, self.score_cap, row_tiles)
+            wv = self.nkv * self.d if self.talks else self.d
+            keys = min(ctx.max_context, window + self.keep_first + 32) if window else ctx.max_context
+            splits = kernels.attn_wide_splits(items.numel() // 4, (wv + 255) // 256, keys) if row_tiles == 1 else 1
+            part = part_ml = None
+            if splits > 1:
+                part = ws.buffer("attn_wide.part", tokens * self.nq * splits, wv, torch.float32)
+                part_ml = ws.buffer("attn_wide.part_ml", tokens * self.nq * splits, 2, torch.float32)
+            kernels.attn_wide(q, each, self.nq, self.nkv, self.d, wv, self.talks, cache.keys, cache.values, ctx.positions,
+                              ctx.token_entry, table, items, hp, self.scale, window, self.keep_first, self.sink,
+                              self.score_cap, row_tiles, splits, part, part_ml)
         else:
             kernels.attn_generic(q, each, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
                                  ctx.token_entry, table, self.scale, window, sink=self.sink, softcap=self.score_cap,

@@ -166,9 +166,15 @@ class LatentAttention(PagedAttention):
                 flat, hp = kernels.attn_wide_items(ctx.entries, self.nq, 1, row_tiles)
                 ctx.extras[key] = (ctx.to_device(flat), hp, row_tiles)
             items, hp, row_tiles = ctx.extras[key]
-            kernels.attn_wide(q, o, self.nq, 1, self.d, (self.rank + 15) // 16 * 16, False, cache.keys, cache.values,
-                              ctx.positions, ctx.token_entry, table, items, hp, self.scale, 0, 0, self.sink, self.score_cap,
-                              row_tiles)
+            wv = (self.rank + 15) // 16 * 16
+            splits = kernels.attn_wide_splits(items.numel() // 4, (wv + 255) // 256, ctx.max_context) if row_tiles == 1 else 1
+            part = part_ml = None
+            if splits > 1:
+                part = ws.buffer("attn_wide.part", tokens * self.nq * splits, self.d, torch.float32)
+                part_ml = ws.buffer("attn_wide.part_ml", tokens * self.nq * splits, 2, torch.float32)
+            kernels.attn_wide(q, o, self.nq, 1, self.d, wv, False, cache.keys, cache.values, ctx.positions,
+                              ctx.token_entry, table, items, hp, self.scale, 0, 0, self.sink, self.score_cap, row_tiles,
+                              splits, part, part_ml)
         else:
             o = ws.buffer("latent.rows", tokens, self.nq * self.d, torch.float32)
             kernels.attn_generic(q, o, self.nq, 1, self.d, cache.keys, cache.values, ctx.positions, ctx.token_entry,

@@ -288,10 +288,16 @@ def test_kept_first_tokens_window_sinks_and_mixed_heads(case, dtype, needle):
         def __init__(self, first_row, count):
             self.first_row, self.count = first_row, count
     step_entries = [E(0, portion)] + [E(portion + i, 1) for i in range(len(lens) - 1)]
-    paths = ["generic"] + (["wide", "wide4"] if kernels.attn_wide_takes(q, kc, d) else [])
+    paths = ["generic"] + (["wide", "wide4", "wide in splits"] if kernels.attn_wide_takes(q, kc, d) else [])
     assert dtype != torch.bfloat16 or bs % 16 or d % 16 or "wide" in paths
     for path in paths:
         row_tiles = 4 if path == "wide4" else 1
+        splits = 3 if path == "wide in splits" else 1
+        scratch = {}
+        if splits > 1:   # (filled with NaN: every sum that is merged must have been written)
+            scratch = dict(n_splits=splits,
+                           part=torch.full((len(positions) * nq * splits, nkv * d), float("nan"), device=DEV),
+                           part_ml=torch.full((len(positions) * nq * splits, 2), float("nan"), device=DEV))
         each = torch.full((len(positions), nq * nkv * d), float("nan"), dtype=torch.float32, device=DEV)
         if path == "generic":
             kernels.attn_generic(q, each, nq, nkv, d, kc, vc, ints(positions), ints(entry), table.to(DEV), scale, window,
@@ -299,7 +305,7 @@ def test_kept_first_tokens_window_sinks_and_mixed_heads(case, dtype, needle):
         else:
             flat, hp = kernels.attn_wide_items(step_entries, nq, nkv, row_tiles)
             kernels.attn_wide(q, each, nq, nkv, d, nkv * d, True, kc, vc, ints(positions), ints(entry), table.to(DEV),
-                              ints(flat), hp, scale, window, keep, sink.to(DEV), row_tiles=row_tiles)
+                              ints(flat), hp, scale, window, keep, sink.to(DEV), row_tiles=row_tiles, **scratch)
         out = torch.full((len(positions), nq * d), float("nan"), dtype=dtype, device=DEV)
         kernels.head_mix(each, mix, out, nq, nkv, d, dv, d, 0.8)
         got = out.cpu().to(F64).view(-1, nq, d)
@@ -317,7 +323,7 @@ def test_kept_first_tokens_window_sinks_and_mixed_heads(case, dtype, needle):
         if path != "generic":   # a head's own values alone, as the part asks for them without mixed heads
             own = torch.full((len(positions), nq * d), float("nan"), dtype=torch.float32, device=DEV)
             kernels.attn_wide(q, own, nq, nkv, d, d, False, kc, vc, ints(positions), ints(entry), table.to(DEV),
-                              ints(flat), hp, scale, window, keep, sink.to(DEV), row_tiles=row_tiles)
+                              ints(flat), hp, scale, window, keep, sink.to(DEV), row_tiles=row_tiles, **scratch)
             got, row = own.cpu().to(F64).view(-1, nq, d), 0
             for r, n in enumerate(lens):
                 rows = portion if r == 0 else 1
