@@ -15,21 +15,22 @@ namespace {
 template <typename TM, typename TY>
 __global__ void head_mix_kernel(const float* __restrict__ x, const TM* __restrict__ mix, TY* __restrict__ y,
                                 int64_t y_stride, int heads, int kv_heads, int d, int dv, int out_d, float scale) {
-    extern __shared__ float m_s[];   // [heads, heads]
-    for (int i = threadIdx.x; i < heads * heads; i += blockDim.x) m_s[i] = to_f32<TM>(mix[i]);
+    // a workgroup a (token, head): that head's row of the mixing matrix in LDS
+    extern __shared__ float m_s[];   // [heads]
+    const int t = blockIdx.x, h = blockIdx.y;
+    for (int i = threadIdx.x; i < heads; i += blockDim.x) m_s[i] = to_f32<TM>(mix[h * heads + i]);
     __syncthreads();
-    const int t = blockIdx.x;
     const int group = heads / kv_heads;
-    const float* row = x + static_cast<int64_t>(t) * heads * kv_heads * d;
-    TY* dst = y + static_cast<int64_t>(t) * y_stride;
-    for (int i = threadIdx.x; i < heads * out_d; i += blockDim.x) {
-        const int h = i / out_d, e = i % out_d;
+    const float* col0 = x + static_cast<int64_t>(t) * heads * kv_heads * d + static_cast<int64_t>(h / group) * d;
+    TY* dst = y + static_cast<int64_t>(t) * y_stride + static_cast<int64_t>(h) * out_d;
+    for (int e = threadIdx.x; e < out_d; e += blockDim.x) {
         float sum = 0.f;
         if (e < dv) {
-            const float* col = row + static_cast<int64_t>(h / group) * d + e;
-            for (int g = 0; g < heads; ++g) sum = fmaf(m_s[h * heads + g], col[static_cast<int64_t>(g) * kv_heads * d], sum);
+            const float* col = col0 + e;
+#pragma unroll 4
+            for (int g = 0; g < heads; ++g) sum = fmaf(m_s[g], col[static_cast<int64_t>(g) * kv_heads * d], sum);
         }
-        dst[i] = from_f32<TY>(sum * scale);
+        dst[e] = from_f32<TY>(sum * scale);
     }
 }
 
@@ -43,12 +44,13 @@ extern "C" int pulse_head_mix(const float* x, const void* mix, int mix_dtype, vo
     PULSE_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && d > 0, "head_mix: bad sizes");
     PULSE_REQUIRE(dv > 0 && dv <= d && out_d >= dv && y_stride >= static_cast<int64_t>(heads) * out_d,
                   "head_mix: bad widths (dv %d, d %d, out %d)", dv, d, out_d);
-    PULSE_REQUIRE(heads <= 128, "head_mix: at most 128 heads, got %d", heads);
+    PULSE_REQUIRE(heads < 65536, "head_mix: too many heads (%d)", heads);
     PULSE_REQUIRE(x && mix && y && pulse_dtype_ok(mix_dtype) && pulse_dtype_ok(y_dtype), "head_mix: bad arguments");
     if (tokens == 0) return 0;
-    const size_t lds = sizeof(float) * heads * heads;
+    const size_t lds = sizeof(float) * heads;
+    const int threads = out_d >= 256 ? 256 : (out_d + 63) / 64 * 64;
     PULSE_DISPATCH_DTYPE(mix_dtype, TM, PULSE_DISPATCH_DTYPE(y_dtype, TY,
-        hipLaunchKernelGGL((head_mix_kernel<TM, TY>), dim3(tokens), dim3(256), lds, stream, x, static_cast<const TM*>(mix),
+        hipLaunchKernelGGL((head_mix_kernel<TM, TY>), dim3(tokens, heads), dim3(threads), lds, stream, x, static_cast<const TM*>(mix),
                            static_cast<TY*>(y), y_stride, heads, kv_heads, d, dv, out_d, scale)));
     PULSE_LAUNCH_CHECK("head_mix");
     return 0;

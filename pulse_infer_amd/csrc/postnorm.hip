@@ -128,12 +128,22 @@ __device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + lo
 
 template <typename T, typename TP>
 __global__ void xielu_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, const TP* __restrict__ pq) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const float a = softplus_f(to_f32<TP>(pq[0])), b = 0.5f + softplus_f(to_f32<TP>(pq[1]));
-    const float z = to_f32<T>(x[i]);
-    const float v = z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z);
-    y[i] = from_f32<T>(v);
+    __shared__ float ab[2];   // the two factors, formed once a workgroup
+    if (threadIdx.x == 0) {
+        ab[0] = softplus_f(to_f32<TP>(pq[0]));
+        ab[1] = 0.5f + softplus_f(to_f32<TP>(pq[1]));
+    }
+    __syncthreads();
+    const float a = ab[0], b = ab[1];
+    const int64_t first = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t i = first + u;
+        if (i < n) {
+            const float z = to_f32<T>(x[i]);
+            y[i] = from_f32<T>(z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z));
+        }
+    }
 }
 
 }  // namespace
@@ -141,7 +151,7 @@ __global__ void xielu_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t
 extern "C" int pulse_xielu(const void* x, void* y, int dtype, int64_t n, const void* pq, int pq_dtype, hipStream_t stream) {
     PULSE_REQUIRE(n >= 0 && x && y && pq && pulse_dtype_ok(dtype) && pulse_dtype_ok(pq_dtype), "xielu: bad arguments");
     if (n == 0) return 0;
-    const int64_t blocks = (n + 255) / 256;
+    const int64_t blocks = (n + 1023) / 1024;   // four neighbouring elements a thread
     PULSE_REQUIRE(blocks < (1ll << 31), "xielu: too many elements");
     PULSE_DISPATCH_DTYPE(dtype, T, PULSE_DISPATCH_DTYPE(pq_dtype, TP,
         hipLaunchKernelGGL((xielu_kernel<T, TP>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
