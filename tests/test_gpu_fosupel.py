@@ -399,7 +399,7 @@ def test_turned_rows_the_walk_and_the_gated_head_norm(dtype, heads, d, dv, dims,
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,d,dr,dv,rank,bs", [(3, 16, 8, 24, 40, 16), (2, 32, 16, 16, 24, 4), (4, 64, 32, 64, 128, 16),
-                                                    (1, 8, 2, 5, 13, 16), (8, 64, 64, 128, 512, 16)])
+                                                    (1, 8, 2, 5, 13, 16), (8, 64, 64, 128, 512, 16), (24, 16, 8, 8, 40, 16)])
 def test_latent_attention_from_its_projections_on(dtype, heads, d, dr, dv, rank, bs):
     """The latent row normed and stored with the turned key part, the queries taken into the latent space, attention
     over one kv head with sinks, the values taken out again and gated: a portion of request 0 beside single tokens,
@@ -624,6 +624,94 @@ def test_a_long_prompt_far_beyond_the_windows(runners, plain, dtype):
     runner = runners(name, dtype, 16, tokens=512)
     agree(run_alone(runner, ids, [400]), want, dtype, "whole", calls)
     agree(run_alone(runner, ids, [150, 190] + [1] * 60), want, dtype, "decoded tail", calls)
+
+
+# ------------------------------------------------------------------------------------ seeded random configurations
+def random_config(rng):
+    """Layers drawn one by one, in any order: head sizes that are no multiples of 16, keys wider or narrower than values,
+    any grouping of heads (more than 16 a kv head too), windows from one token on and none, kept tokens beyond the
+    window, rotations on a part of a head, on all of it and none, with and without scaled frequencies, latent rows that
+    are no multiples of 8, routers that choose all their experts, layers without a feed-forward, loops over any stretch
+    of the layers (also none, and a single pass)."""
+    width = rng.choice([64, 96, 160, 256])
+    layers = []
+    for _ in range(rng.choice([1, 2, 3])):
+        if rng.random() < 0.6:
+            groups, share = rng.choice([1, 2, 3]), rng.choice([1, 2, 3, 4, 18])
+            dim = rng.choice([16, 24, 32, 48, 64])
+            dims = rng.choice([x for x in (0, 2, 8, 16, 24, dim) if x <= dim])
+            window = rng.choice([1, 5, 16, 33, 100, None])
+            l = left(groups * share, groups, dim, rng.choice([8, 16, 40, 48, 64]), window, rng.choice([0, 1, 4, 20]),
+                     rot(rng.choice([100.0, 1e4, 5e5]), dims, rng.choice([None, 1.0, 8.0])) if dims else None,
+                     rng.choice([0.1, dim ** -0.5, 0.5]))
+            heads, rdim = rng.choice([1, 2, 3, 5]), rng.choice([16, 24, 32, 64])
+            rdims = rng.choice([x for x in (0, 4, 16, rdim) if x <= rdim])
+            r = right(heads, rdim, rng.choice([16, 20, 32, 72]), [rng.choice([0.9, 0.97, 0.99, 1.0]) for _ in range(heads)],
+                      rot(rng.choice([100.0, 1e4]), rdims) if rdims else None)
+            mixer = parallel(l, r, rng.choice([0.5, 1.0, 1.5]), rng.choice([0.7, 1.0]))
+        else:
+            mixer = latent(rng.choice([1, 2, 4, 20]), rng.choice([8, 16, 24, 40]), rng.choice([2, 8, 16, 32]),
+                           rng.choice([8, 16, 20, 48]), rng.choice([12, 24, 32, 64, 100]), rng.choice([1e3, 1e4, 1e6]),
+                           rng.choice([0.1, 0.2]))
+        kind = rng.choice(["none", "dense", "moe", "moe"])
+        if kind == "none":
+            mlp = None
+        elif kind == "dense":
+            mlp = dense(rng.choice([32, 100, 256]))
+        else:
+            experts = rng.choice([1, 2, 4, 9])
+            mlp = moe(experts, rng.randint(1, min(4, experts)), rng.choice([32, 40, 64, 100]), rng.choice([None, 48, 128]))
+        layers.append(layer(mixer, mlp))
+    loop = None
+    if rng.random() < 0.7:
+        start = rng.randint(0, len(layers))
+        loop = (start, rng.randint(start, len(layers)), rng.choice([1, 2, 3]))
+    return config(rng.choice([257, 300, 1000]), width, rng.choice([1e-6, 1e-5]), rng.choice([0.3, 1.0, 1.4]),
+                  rng.choice([0.0, 5.0, 50.0]), loop, layers)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations(tmp_path, seed):
+    """Whole, with the last 20 tokens one by one, and in portions of 2 to 70 tokens, in 32-bit and in bfloat16."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    import random
+
+    from pulse_infer_amd.config import FosupelConfig
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.weights import write_model_folder
+
+    rng = random.Random(9000 + seed)
+    cfg = random_config(rng)
+    length = rng.choice([90, 150])
+    folder = write_model_folder(FosupelConfig.from_dict(cfg), str(tmp_path / "m"), seed=seed)
+    oracle = P.PlainFosupel.from_folder(folder)
+    ids = token_ids(cfg["vocab"], length, seed=seed)
+    want = oracle.logits(ids)
+    calls = Calls(set((oracle.router_margins(ids) < CLOSE_CALL).nonzero().flatten().tolist()), oracle.fragile_positions(ids))
+    what = f"{cfg} length {length}"
+    for dtype in ("float32", "bfloat16"):
+        _, model = load_model(folder, mode=dtype)
+        runner = ModelRunner(model, page_size=16, num_pages=16, max_requests=4)
+        whole = run_alone(runner, ids, [length])
+        agree(whole, want, dtype, f"whole: {what}", calls)
+        tail = run_alone(runner, ids, [length - 20] + [1] * 20)
+        agree(tail, want, dtype, f"tail: {what}", calls)
+        cuts, left_over, sizes = [], length, [40, 2, 17, 3, 70, 5, 19]
+        while left_over:
+            n = min(sizes[len(cuts) % len(sizes)], left_over)
+            cuts.append(n)
+            left_over -= n
+        portions = run_alone(runner, ids, cuts)
+        agree(portions, want, dtype, f"portions {cuts}: {what}", calls)
+        # however the prompt is cut: the same logits (in 32-bit only the fragile positions are left out; in bfloat16
+        # another cut may also tip a router's close call)
+        left_out = Calls(set(), calls.fragile) if dtype == "float32" else calls
+        agree(tail, whole, dtype, f"tail against whole: {what}", left_out)
+        agree(portions, whole, dtype, f"portions against whole: {what}", left_out)
+        del runner, model
+    torch.cuda.empty_cache()
 
 
 # ------------------------------------------------------------------------------------------------ long decoding
