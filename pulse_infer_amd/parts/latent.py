@@ -6,8 +6,9 @@ position, are all that is cached.  Head h's key is [W_uk,h c | k_rot] (the turne
 value W_uv,h c; scores are (q . key) * scale over all earlier tokens, softmax with an optional sink per head; the
 heads' results, side by side, are multiplied element by element by sigmoid(Wg x) (optional) and projected by Wo.
 
-Scores and weighted sums are linear in c, so the part works in the latent space and the paged attention kernels of
-``attention`` serve it unchanged: one kv head whose stored key is [c | k_rot] and whose stored value is c, query head
+Scores and weighted sums are linear in c, so the part works in the latent space and paged attention kernels serve it
+as they are (those of ``attention`` where they are compiled for rows this wide, else ``pulse_attn_wide``, else the
+generic one): one kv head whose stored key is [c | k_rot] and whose stored value is c, query head
 h = [W_uk,h^T q_plain,h | q_rot,h], and W_uv,h applied to the weighted sum of latent rows afterwards.  Keys and values
 are stored ``stored`` = latent_dim + rotary_dim (rounded up to 16) channels wide, the rest zeros.
 
@@ -15,8 +16,9 @@ Parameters: ``hidden_size``, ``num_heads``, ``head_dim`` (plain channels of a he
 ``latent_dim``, ``scale``, ``norm_eps``, ``position`` (a rotary encoding of ``rotary_dim`` channels), ``sink``,
 ``output_gate`` (True: by channel), ``names``, ``out_scale``.
 
-Kernels: ``pulse_latent_rows`` (norm of the latent row, turns, page write), ``pulse_latent_absorb`` (queries into the
-latent space), the attention kernels, ``pulse_latent_expand`` (values out of the latent space, gate).  It answers the
+Kernels: ``pulse_latent_rows`` (norm of the latent row, turns, page write), ``pulse_heads_product`` (bfloat16: both
+products a head on the matrix cores) or ``pulse_latent_absorb`` / ``pulse_latent_expand`` (queries into the latent
+space, values out of it with the gate), and the attention kernels between them.  It answers the
 protocol of a branch of ``side_by_side``.
 """
 from __future__ import annotations
