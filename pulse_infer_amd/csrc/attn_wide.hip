@@ -101,18 +101,27 @@ __global__ __launch_bounds__(256, R == 1 ? 3 : 1) void attn_wide_kernel(const bf
 
     const int per_split = (nsteps + a.n_splits - 1) / a.n_splits;
     const int step0 = static_cast<int>(blockIdx.z) * per_split, step1 = min(nsteps, step0 + per_split);
+    // the page numbers of a step are asked for a step ahead, so that their trip lies behind the step in hand
+    auto lookup = [&](int st, int t) __attribute__((always_inline)) {
+        const int ub = st * 32 + 16 * t;
+        const int jb = ub < nfirst ? ub : lo16 + ub - nfirst;
+        const int pi = jb / a.page_size;
+        return (st < step1 && ub < total && pi < a.bt_width) ? bt[pi] : -1;
+    };
+    int ahead[2] = {lookup(step0 + wave, 0), lookup(step0 + wave, 1)};
     for (int step = step0 + wave; step < step1; step += 4) {
         int page[2], off[2], jbase[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int ub = step * 32 + 16 * t;
             const int jb = ub < nfirst ? ub : lo16 + ub - nfirst;
-            const int pi = jb / a.page_size;
-            const int p = (ub < total && pi < a.bt_width) ? bt[pi] : -1;
+            const int p = ahead[t];
             page[t] = (p >= 0 && p < a.num_pages) ? p : -1;
             off[t] = jb % a.page_size;
             jbase[t] = jb;
         }
+        ahead[0] = lookup(step + 4, 0);
+        ahead[1] = lookup(step + 4, 1);
         // S^T: keys x rows, for every row tile from the same key operands
         f32x4 s[R][2];
 #pragma unroll
