@@ -35,6 +35,13 @@ struct ScanArgs {
                           //    entry's last piece leaves the state in the slot
     const int* pieces;    // modes 1, 2: [pieces][4] = first row, tokens, entry, 1 (entry's first) | 2 (entry's last)
     float* scratch;       // [pieces, heads, d, dv]
+    // q and k may be turned by the tokens' positions as they are fetched (float32, before anything else is done with
+    // them): the first `rot` channels of every head, pairs (i, i + rot / 2) with pairing 1 or (2i, 2i + 1) with 0, by
+    // the tables cos_t / sin_t [T, rot / 2]; k is multiplied by k_scale after the turn
+    const float* cos_t;
+    const float* sin_t;
+    int rot, pairing;
+    float k_scale;
 };
 
 __device__ __forceinline__ float activate(float z, int act) { return act == 1 ? z / (1.0f + expf(-z)) : z; }
@@ -127,8 +134,26 @@ __global__ __launch_bounds__(SCAN_THREADS) void lightning_scan_kernel(const TX* 
             qr[u] = kr[u] = 0.f;
             if (tt < nb && i < a.d) {
                 const TX* row = x + static_cast<int64_t>(row0 + t0 + tt) * a.x_stride;
-                if (outputs) qr[u] = to_f32<TX>(row[a.q0 + h * a.d + i]);
-                kr[u] = to_f32<TX>(row[a.k0 + h * a.d + i]);
+                const TX* qh = row + a.q0 + h * a.d;
+                const TX* kh = row + a.k0 + h * a.d;
+                float qv = outputs ? to_f32<TX>(qh[i]) : 0.f, kv = to_f32<TX>(kh[i]);
+                if (i < a.rot) {
+                    const int half = a.rot / 2;
+                    int pair, freq;
+                    bool first;
+                    if (a.pairing == 1) { first = i < half; pair = first ? i + half : i - half; freq = first ? i : i - half; }
+                    else { first = (i & 1) == 0; pair = i ^ 1; freq = i >> 1; }
+                    const int64_t at = static_cast<int64_t>(row0 + t0 + tt) * half + freq;
+                    const float c = a.cos_t[at], sn = a.sin_t[at];
+                    const float ko = to_f32<TX>(kh[pair]);
+                    kv = first ? kv * c - ko * sn : kv * c + ko * sn;
+                    if (outputs) {
+                        const float qo = to_f32<TX>(qh[pair]);
+                        qv = first ? qv * c - qo * sn : qv * c + qo * sn;
+                    }
+                }
+                qr[u] = qv;
+                kr[u] = kv * a.k_scale;
             }
         }
 #pragma unroll
@@ -275,11 +300,15 @@ int launch_scan_d(int r, const void* x, float* out, float* state, const float* d
 // mode 0: a workgroup walks an entry.  Modes 1 and 2 walk `n_pieces` pieces of entries (see ScanArgs): a long portion
 // is walked twice, first every piece from a zero state (mode 1), then, after pulse_lightning_combine has turned what the
 // pieces left into the states between them, every piece with its outputs (mode 2); all pieces run at the same time.
-extern "C" int pulse_lightning_scan(const void* x, int x_dtype, int64_t x_stride, int q0, int k0, int v0, float* out,
-                                    int64_t o_stride, float* state, int slots, const float* decay,
-                                    const int* entry_first_row, const int* entry_start, const int* entry_slot,
-                                    int entries, int heads, int d, int dv, int act, int row_groups, int mode,
-                                    const int* pieces, int n_pieces, float* scratch, hipStream_t stream) {
+// cos_t / sin_t (float32 [T, rot / 2]; null: no turn), rot, pairing, k_scale: see ScanArgs.
+extern "C" int pulse_lightning_scan_turned(const void* x, int x_dtype, int64_t x_stride, int q0, int k0, int v0, float* out,
+                                           int64_t o_stride, float* state, int slots, const float* decay,
+                                           const int* entry_first_row, const int* entry_start, const int* entry_slot,
+                                           int entries, int heads, int d, int dv, int act, int row_groups, int mode,
+                                           const int* pieces, int n_pieces, float* scratch, const float* cos_t,
+                                           const float* sin_t, int rot, int pairing, float k_scale, hipStream_t stream) {
+    PULSE_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= d && (rot == 0 || (cos_t && sin_t && act == 0)) &&
+                  (pairing == 0 || pairing == 1), "lightning_scan: bad rotation (%d of %d channels)", rot, d);
     PULSE_REQUIRE(mode >= 0 && mode <= 2 && (mode == 0 || (pieces && scratch && n_pieces > 0)),
                   "lightning_scan: a walk in pieces needs its pieces and scratch");
     PULSE_REQUIRE(entries >= 0 && heads > 0 && d > 0 && dv > 0 && slots > 0, "lightning_scan: bad sizes");
@@ -295,6 +324,7 @@ extern "C" int pulse_lightning_scan(const void* x, int x_dtype, int64_t x_stride
     a.heads = heads; a.d = d; a.dv = dv; a.x_stride = x_stride; a.o_stride = o_stride;
     a.q0 = q0; a.k0 = k0; a.v0 = v0; a.act = act;
     a.mode = mode; a.pieces = pieces; a.scratch = scratch;
+    a.cos_t = cos_t; a.sin_t = sin_t; a.rot = cos_t ? rot : 0; a.pairing = pairing; a.k_scale = k_scale;
     if (mode != 0) entries = n_pieces;   // workgroups along x
     int rc = 0;
 #define PULSE_SCAN_CASE(DD)                                                                                            \
@@ -309,6 +339,16 @@ extern "C" int pulse_lightning_scan(const void* x, int x_dtype, int64_t x_stride
     if (rc) return rc;
     PULSE_LAUNCH_CHECK("lightning_scan");
     return 0;
+}
+
+extern "C" int pulse_lightning_scan(const void* x, int x_dtype, int64_t x_stride, int q0, int k0, int v0, float* out,
+                                    int64_t o_stride, float* state, int slots, const float* decay,
+                                    const int* entry_first_row, const int* entry_start, const int* entry_slot,
+                                    int entries, int heads, int d, int dv, int act, int row_groups, int mode,
+                                    const int* pieces, int n_pieces, float* scratch, hipStream_t stream) {
+    return pulse_lightning_scan_turned(x, x_dtype, x_stride, q0, k0, v0, out, o_stride, state, slots, decay, entry_first_row,
+                                       entry_start, entry_slot, entries, heads, d, dv, act, row_groups, mode, pieces,
+                                       n_pieces, scratch, nullptr, nullptr, 0, 0, 1.0f, stream);
 }
 
 extern "C" int pulse_lightning_combine(float* scratch, const float* state, const float* decay, const int* pieces,

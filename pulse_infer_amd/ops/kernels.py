@@ -1038,15 +1038,27 @@ def lightning_scan(x: torch.Tensor, q0: int, k0: int, v0: int, out: torch.Tensor
                    decay: torch.Tensor, entry_first_row: torch.Tensor, entry_start: torch.Tensor,
                    entry_slot: torch.Tensor, heads: int, d: int, dv: int, activation: str = "silu",
                    row_groups: int = 1, pieces: Optional[torch.Tensor] = None,
-                   scratch: Optional[torch.Tensor] = None) -> None:
+                   scratch: Optional[torch.Tensor] = None, turn: Optional[tuple] = None, key_scale: float = 1.0) -> None:
     """For every entry of the step, token by token: S <- decay_h S + k v^T, out = S^T q, per head, in float32;
     S [slots, heads, d, dv] is the state of the entry's slot, zero when the entry starts at position 0.
 
     ``pieces`` (int32 [n, 4]: first row, tokens, entry, 1 for an entry's first piece | 2 for its last; an entry's
     pieces in order and next to each other) with ``scratch`` (float32 [n, heads, d, dv]): the entries are walked in
     these pieces, all at the same time: every piece from a zero state, then the states between the pieces from what
-    each left, then every piece again with its outputs."""
+    each left, then every piece again with its outputs.
+
+    ``turn`` = (cos, sin, rotary_dim, pairing): q and k are turned by the tokens' tables (float32 [T, rotary_dim / 2])
+    as they are fetched, in float32 (activation "none" only); ``key_scale``: k is multiplied by it after the turn."""
     _gpu("lightning_scan", x, out, state, decay, entry_first_row, entry_start, entry_slot)
+    cos = sin = None
+    rot = pairing = 0
+    if turn is not None and turn[0] is not None and turn[2]:
+        cos, sin, rot, pairing = turn
+        _gpu("lightning_scan", cos, sin)
+        _need(activation == "none", "lightning_scan: q and k are turned as they are projected (activation 'none')")
+        for t in (cos, sin):
+            _need(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (x.shape[0], rot // 2),
+                  f"lightning_scan: the tables must be contiguous float32 [{x.shape[0]}, {rot // 2}]")
     entries = entry_start.numel()
     _need(x.dim() == 2 and x.stride(1) == 1, "lightning_scan: x must be a matrix with contiguous rows")
     _need(out.dtype == torch.float32 and out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == x.shape[0]
@@ -1063,11 +1075,11 @@ def lightning_scan(x: torch.Tensor, q0: int, k0: int, v0: int, out: torch.Tensor
     _need(min(q0, k0, v0) >= 0 and max(q0, k0) + heads * d <= width and v0 + heads * dv <= width,
           "lightning_scan: q, k or v columns lie outside x")
     def walk(mode: int, n_pieces: int) -> None:
-        call("pulse_lightning_scan", _ptr(x), _i32(_tag(x, "lightning_scan")), _i64(x.stride(0)), _i32(q0), _i32(k0),
+        call("pulse_lightning_scan_turned", _ptr(x), _i32(_tag(x, "lightning_scan")), _i64(x.stride(0)), _i32(q0), _i32(k0),
              _i32(v0), _ptr(out), _i64(out.stride(0)), _ptr(state), _i32(state.shape[0]), _ptr(decay),
              _ptr(entry_first_row), _ptr(entry_start), _ptr(entry_slot), _i32(entries), _i32(heads), _i32(d), _i32(dv),
              _i32(1 if activation == "silu" else 0), _i32(row_groups), _i32(mode), _ptr(pieces), _i32(n_pieces),
-             _ptr(scratch), _stream())
+             _ptr(scratch), _ptr(cos), _ptr(sin), _i32(rot), _i32(pairing), _f32(key_scale), _stream())
 
     if pieces is None:
         walk(0, 0)

@@ -17,9 +17,9 @@ Variations ("retention" is the combination of all of them): ``position``: a posi
 rotation turns the first channels of every head of q and k (activation "none" only); ``key_scale``: a factor on k,
 after the rotation; ``norm``: "all" (default: the heads of a token normed together) or "head" (every head divided by
 its own root mean square); ``norm_weight`` (default True; False: the norm has no weight and no tensor);
-``gate_activation``: "sigmoid" (default) or "silu".  With a rotation or a key factor q, k and v go from the
-projection's output into float32 rows first (``pulse_rotate_qk_rows``), which the walk reads: nothing behind the
-projection is rounded before it enters the recurrence.
+``gate_activation``: "sigmoid" (default) or "silu".  A rotation and a key factor are applied in float32, by the walk
+itself as it fetches q and k (few tokens) or into float32 rows of their own that the walk then reads
+(``pulse_rotate_qk_rows``, long portions): nothing behind the projection is rounded before it enters the recurrence.
 
 The part keeps a ``StateSpec`` per run.  It also answers the protocol of a branch of ``side_by_side``:
 ``inner_width``, ``out_weight()`` and ``forward_inner(x, ctx, cache, out)``.
@@ -114,6 +114,7 @@ class LightningAttention(Part):
         self.inner_width = self.heads * self.dv
 
     records_cleanly = True   # slots, starts and rows are read on the device
+    TURN_AHEAD_TOKENS = 256  # steps of at least this many tokens turn q and k in a launch of their own
 
     def cache_spec(self) -> StateSpec:
         return StateSpec((self.heads, self.d, self.dv), "float32")
@@ -144,16 +145,23 @@ class LightningAttention(Part):
             walkers = pieces.numel() // 4
             scratch = ws.buffer("lightning.pieces", walkers, self.heads * self.d * self.dv, torch.float32)
         groups = kernels.lightning_row_groups(walkers, self.heads, self.d, self.dv)
-        rows = y
-        if self.position is not None or self.key_scale != 1.0:
-            tables = ctx.position_product(self.position, self.encodings) if self.position is not None else None
+        # A rotation and a key factor, in float32 either way: for few tokens the walk applies them itself as it fetches q
+        # and k (a launch less: 47 + 44 -> 49 us for 8 decoded tokens of three layers of 16 heads of 128); long portions,
+        # which are walked twice in pieces, get turned float32 rows of their own first (2,048 tokens: 114 + 439 us
+        # against 834 with the turn inside both walks).
+        turn, rows, scale = None, y, self.key_scale
+        if self.position is not None:
+            tables = ctx.position_product(self.position, self.encodings)
+            turn = (tables.cos, tables.sin, tables.rotary_dim, tables.pairing)
+        if tokens >= self.TURN_AHEAD_TOKENS and (turn is not None or scale != 1.0):
             rows = ws.buffer("lightning.rows", tokens, 2 * hd + hv, torch.float32)
             kernels.rotate_qk_rows(y, 0, hd, 2 * hd, rows, self.heads, self.d, self.dv,
-                                   tables.cos if tables is not None else None, tables.sin if tables is not None else None,
-                                   tables.rotary_dim if tables is not None else 0,
-                                   tables.pairing if tables is not None else 0, self.key_scale)
+                                   turn[0] if turn else None, turn[1] if turn else None, turn[2] if turn else 0,
+                                   turn[3] if turn else 0, scale)
+            turn, scale = None, 1.0
         kernels.lightning_scan(rows, 0, hd, 2 * hd, o, cache.state, self.decay, ctx.entry_first_row, ctx.entry_start,
-                               ctx.entry_slot, self.heads, self.d, self.dv, self.activation, groups, pieces, scratch)
+                               ctx.entry_slot, self.heads, self.d, self.dv, self.activation, groups, pieces, scratch,
+                               turn=turn, key_scale=scale)
         gate = y[:, 2 * hd + hv:]
         if self.norm_over == "all" and self.norm_weight is not None and self.gate_activation == "sigmoid":
             kernels.gated_rmsnorm(o, self.norm_weight, gate, out, self.eps, self.out_scale)

@@ -368,7 +368,8 @@ def test_turned_rows_the_walk_and_the_gated_head_norm(dtype, heads, d, dv, dims,
     decay, base, eps = [0.5, 1.0, 0.97, 0.999][:heads], 700.0, 1e-5
     counts, starts, slot_of = [37, 20, 1], [12, 0, 300], [3, 0, 4]
     hd, hv = heads * d, heads * dv
-    state = torch.full((5, heads, d, dv), float("nan"), dtype=torch.float32, device=DEV)
+    state0 = torch.full((5, heads, d, dv), float("nan"), dtype=torch.float32, device=DEV)
+    state1 = state0.clone()
     wants, rows_of = [], []
     for r, (n, s0) in enumerate(zip(counts, starts)):
         total = s0 + n
@@ -382,29 +383,39 @@ def test_turned_rows_the_walk_and_the_gated_head_norm(dtype, heads, d, dv, dims,
         rows_of.append(y)
     inv = base ** (-2.0 * torch.arange(max(dims, 2) // 2, dtype=F64) / max(dims, 2))
 
-    def run(rows, positions, first_row, start, slots):
+    def run(rows, positions, first_row, start, slots, state=None, fused=False):
+        state = state0 if state is None else state
         tokens = rows.shape[0]
         cos = sin = None
         if dims:
             angle = torch.tensor(positions, dtype=F64).view(-1, 1) * inv.view(1, -1)
             cos, sin = torch.cos(angle).float().to(DEV).contiguous(), torch.sin(angle).float().to(DEV).contiguous()
-        wide = torch.full((tokens, 2 * hd + hv), float("nan"), dtype=torch.float32, device=DEV)
-        kernels.rotate_qk_rows(rows, 0, hd, 2 * hd, wide, heads, d, dv, cos, sin, dims, 1 if pairing == "half" else 0, d ** -0.5)
         o = torch.full((tokens, hv), float("nan"), dtype=torch.float32, device=DEV)
-        kernels.lightning_scan(wide, 0, hd, 2 * hd, o, state, torch.tensor(decay, device=DEV), ints(first_row), ints(start),
-                               ints(slots), heads, d, dv, "none", kernels.lightning_row_groups(len(start), heads, d, dv))
+        groups = kernels.lightning_row_groups(len(start), heads, d, dv)
+        if fused:    # the walk turns and scales as it fetches
+            kernels.lightning_scan(rows, 0, hd, 2 * hd, o, state, torch.tensor(decay, device=DEV), ints(first_row),
+                                   ints(start), ints(slots), heads, d, dv, "none", groups,
+                                   turn=(cos, sin, dims, 1 if pairing == "half" else 0), key_scale=d ** -0.5)
+        else:        # turned float32 rows of their own first
+            wide = torch.full((tokens, 2 * hd + hv), float("nan"), dtype=torch.float32, device=DEV)
+            kernels.rotate_qk_rows(rows, 0, hd, 2 * hd, wide, heads, d, dv, cos, sin, dims, 1 if pairing == "half" else 0,
+                                   d ** -0.5)
+            kernels.lightning_scan(wide, 0, hd, 2 * hd, o, state, torch.tensor(decay, device=DEV), ints(first_row),
+                                   ints(start), ints(slots), heads, d, dv, "none", groups)
         out = torch.full((tokens, hv), float("nan"), dtype=dtype, device=DEV)
         kernels.group_norm_gate(o, None, rows[:, 2 * hd + hv:], out, heads, eps, 1.3, "silu")
         return out.cpu().to(F64)
 
     # what came before this step: the first and the third request's earlier tokens
-    for r in (0, 2):
-        run(rows_of[r][:starts[r]].contiguous(), list(range(starts[r])), [0, starts[r]], [0], [slot_of[r]])
     step = torch.cat([rows_of[r][starts[r]:] for r in range(3)]).contiguous()
     positions = [p for r in range(3) for p in range(starts[r], starts[r] + counts[r])]
     first_row = [0, counts[0], counts[0] + counts[1], sum(counts)]
-    got = run(step, positions, first_row, starts, slot_of)
-    assert torch.allclose(got, torch.cat(wants), **tol(dtype)), float((got - torch.cat(wants)).abs().max())
+    for state, fused in ((state0, False), (state1, True)):
+        for r in (0, 2):
+            run(rows_of[r][:starts[r]].contiguous(), list(range(starts[r])), [0, starts[r]], [0], [slot_of[r]], state, fused)
+        got = run(step, positions, first_row, starts, slot_of, state, fused)
+        assert torch.allclose(got, torch.cat(wants), **tol(dtype)), (fused, float((got - torch.cat(wants)).abs().max()))
+    assert torch.allclose(state0[[0, 3, 4]], state1[[0, 3, 4]], atol=1e-5, rtol=1e-5)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
